@@ -7,7 +7,15 @@
 // bidirectional block has kv_hi = end of its block; a window of w has
 // kv_lo = max(0, p + 1 - w). The keys of this step are already in the cache.
 // Key position k of row r lies at page block_table[r, k / page_size], offset
-// k % page_size; key cache [pages, Hkv, page_size, hd], value cache [pages, Hkv, hd, page_size].
+// k % page_size; key cache [pages, Hkv, page_size, hd], value cache [pages, Hkv, hdv, page_size]:
+// values may have another size than queries and keys (hdv channels; the output is [n, H hdv]).
+//
+// Two optional terms of the scores, for mixers that encode order by distance instead of by a
+// rotation, and that let a query attend to nothing:
+//  * slopes (fp32 [H]) with positions (int32 [n], the place of every query in its row): the score
+//    of query position i against key position j is lowered by slopes[h] * (i - j);
+//  * a sink: one more term exp(sink_score) in the softmax's denominator that carries no value
+//    (has_sink != 0). The running maximum and sum then start from that term instead of from nothing.
 #include "ka_common.h"
 
 constexpr int ATT_MAX_HD = 512;
@@ -28,7 +36,8 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
                          int max_pages, const int* __restrict__ token_row,
                          const int* __restrict__ kv_lo, const int* __restrict__ kv_hi,
                          T* __restrict__ out, long out_row_stride, float scale, int H, int Hkv,
-                         int hd, int page_size) {
+                         int hd, int hdv, int page_size, const int* __restrict__ positions,
+                         const float* __restrict__ slopes, int has_sink, float sink_score) {
     __shared__ float qs[ATT_MAX_HD];
     __shared__ float ps[KA_WAVE];
     __shared__ long offs[KA_WAVE];   // value cache offset of channel 0 of each key of the chunk
@@ -38,11 +47,13 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
     int lo = kv_lo ? kv_lo[t] : 0, hi = kv_hi[t];
     const T* qp = q + (size_t)t * q_row_stride + (size_t)h * hd;
     for (int d = lane; d < hd; d += KA_WAVE) qs[d] = ka_to_float(qp[d]) * scale;
+    const float slope = slopes ? slopes[h] : 0.f;
+    const int place = slopes ? positions[t] : 0;
     __syncthreads();
     const int* bt = block_table + (size_t)row * max_pages;
     const bool k_vectors = hd % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
     const bool v_vectors = page_size % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % (4 * sizeof(T)) == 0;
-    float m = -INFINITY, l = 0.f;
+    float m = has_sink ? sink_score : -INFINITY, l = has_sink ? 1.f : 0.f;
     float o[ATT_MAX_HD / KA_WAVE];
 #pragma unroll
     for (int i = 0; i < ATT_MAX_HD / KA_WAVE; ++i) o[i] = 0.f;
@@ -54,7 +65,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
         if (valid) {
             int page = bt[key / page_size];
             const T* kp = k_cache + (((long)page * Hkv + kvh) * page_size + key % page_size) * hd;
-            off = ((long)page * Hkv + kvh) * hd * page_size + key % page_size;
+            off = ((long)page * Hkv + kvh) * hdv * page_size + key % page_size;
             float acc = 0.f;
             if (k_vectors) {
                 // four channels with one load, added in the same order as one by one
@@ -67,7 +78,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
             } else {
                 for (int d = 0; d < hd; ++d) acc = fmaf(qs[d], ka_to_float(kp[d]), acc);
             }
-            s = acc;
+            s = slopes ? acc - slope * (float)(place - key) : acc;
         }
         float m_new = fmaxf(m, ka_wave_max(s));
         float corr = expf(m - m_new);  // m = -inf at the first chunk gives 0
@@ -82,7 +93,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
 #pragma unroll
         for (int i = 0; i < ATT_MAX_HD / KA_WAVE; ++i) {
             int d = lane + i * KA_WAVE;
-            if (d < hd) {
+            if (d < hdv) {
                 float acc = o[i] * corr;
                 const T* vd = v_cache + (long)d * page_size;
                 int j = 0;
@@ -103,11 +114,11 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
         }
     }
     float inv = l > 0.f ? 1.0f / l : 0.f;
-    T* op = out + (size_t)t * out_row_stride + (size_t)h * hd;
+    T* op = out + (size_t)t * out_row_stride + (size_t)h * hdv;
 #pragma unroll
     for (int i = 0; i < ATT_MAX_HD / KA_WAVE; ++i) {
         int d = lane + i * KA_WAVE;
-        if (d < hd) op[d] = ka_from_float<T>(o[i] * inv);
+        if (d < hdv) op[d] = ka_from_float<T>(o[i] * inv);
     }
 }
 
@@ -115,8 +126,11 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
                                 const void* v_cache, const int* block_table, int max_pages,
                                 const int* token_row, const int* kv_lo, const int* kv_hi, void* out,
                                 long out_row_stride, float scale, int n, int H, int Hkv, int hd,
-                                int page_size, hipStream_t stream) {
-    KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0, "ka_attention_generic: bad sizes");
+                                int page_size, int hdv, const int* positions, const float* slopes,
+                                int has_sink, float sink_score, hipStream_t stream) {
+    KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0 && hdv > 0, "ka_attention_generic: bad sizes");
+    KA_CHECK(hdv <= ATT_MAX_HD, "ka_attention_generic: value size %d above %d", hdv, ATT_MAX_HD);
+    KA_CHECK(slopes == nullptr || positions != nullptr, "ka_attention_generic: slopes need the queries' positions");
     KA_CHECK(H % Hkv == 0, "ka_attention_generic: %d query heads do not divide into %d kv heads", H, Hkv);
     KA_CHECK(hd <= ATT_MAX_HD, "ka_attention_generic: head size %d above %d", hd, ATT_MAX_HD);
     KA_CHECK(H <= 65535, "ka_attention_generic: too many heads %d", H);
@@ -126,11 +140,13 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
     if (dtype == KA_F32)
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_row_stride,
                            (const float*)k_cache, (const float*)v_cache, block_table, max_pages, token_row, kv_lo,
-                           kv_hi, (float*)out, out_row_stride, scale, H, Hkv, hd, page_size);
+                           kv_hi, (float*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
+                           sink_score);
     else if (dtype == KA_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
                            (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
-                           kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, hd, page_size);
+                           kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
+                           sink_score);
     else
         KA_CHECK(false, "ka_attention_generic: unsupported dtype %d", dtype);
     KA_LAUNCH_CHECK();

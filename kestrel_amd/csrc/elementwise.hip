@@ -312,3 +312,217 @@ KA_API int ka_rope_cache(void* qkv, int dtype, long row_stride, const int* posit
     KA_LAUNCH_CHECK();
     return 0;
 }
+
+// ----------------------------------------------------------------------------
+// Learned position vectors: x[t, :] += table[places[t], :] in fp32 (a place outside the table
+// adds nothing).
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ void add_table_rows_kernel(const T* __restrict__ table, int table_rows, const int* __restrict__ places,
+                                      float* __restrict__ x, int dim) {
+    const int t = blockIdx.x;
+    const int p = places[t];
+    if ((unsigned)p >= (unsigned)table_rows) return;
+    const T* src = table + (size_t)p * dim;
+    float* dst = x + (size_t)t * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] += ka_to_float(src[d]);
+}
+
+KA_API int ka_add_table_rows(const void* table, int table_dtype, int table_rows, const int* places, float* x, int n,
+                             int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0 && table_rows > 0, "ka_add_table_rows: bad sizes n=%d dim=%d rows=%d", n, dim, table_rows);
+    if (n == 0) return 0;
+    dim3 grid(n), block(256);
+    if (table_dtype == KA_F32)
+        hipLaunchKernelGGL(add_table_rows_kernel<float>, grid, block, 0, stream, (const float*)table, table_rows, places, x, dim);
+    else if (table_dtype == KA_BF16)
+        hipLaunchKernelGGL(add_table_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, table_rows, places, x, dim);
+    else
+        KA_CHECK(false, "ka_add_table_rows: unsupported table dtype %d", table_dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// fp32 rows into a range of columns of wider rows of the activation type: dst[t, :dim] = src[t, :]
+// with dst rows `dst_stride` apart (the caller points dst at the first column of the range).
+// Two such calls lay two streams side by side as the input of one linear.
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ void cast_columns_kernel(const float* __restrict__ src, T* __restrict__ dst, long dst_stride, int dim) {
+    const int t = blockIdx.x;
+    const float* s = src + (size_t)t * dim;
+    T* d = dst + (size_t)t * dst_stride;
+    for (int c = threadIdx.x; c < dim; c += blockDim.x) d[c] = ka_from_float<T>(s[c]);
+}
+
+KA_API int ka_cast_columns(const float* src, void* dst, int dst_dtype, long dst_stride, int n, int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0 && dst_stride >= dim, "ka_cast_columns: bad sizes n=%d dim=%d stride=%ld", n, dim, dst_stride);
+    if (n == 0) return 0;
+    dim3 grid(n), block(256);
+    if (dst_dtype == KA_F32)
+        hipLaunchKernelGGL(cast_columns_kernel<float>, grid, block, 0, stream, src, (float*)dst, dst_stride, dim);
+    else if (dst_dtype == KA_BF16)
+        hipLaunchKernelGGL(cast_columns_kernel<bf16_t>, grid, block, 0, stream, src, (bf16_t*)dst, dst_stride, dim);
+    else
+        KA_CHECK(false, "ka_cast_columns: unsupported dtype %d", dst_dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// x += scale * delta over fp32 buffers of one length (a block's branch outputs, summed in delta,
+// enter the residual stream with a weight).
+// ----------------------------------------------------------------------------
+__global__ void add_scaled_kernel(float* __restrict__ x, const float* __restrict__ delta, float scale, long count) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < count) x[i] = fmaf(scale, delta[i], x[i]);
+}
+
+KA_API int ka_add_scaled(float* x, const float* delta, float scale, long count, hipStream_t stream) {
+    KA_CHECK(count >= 0 && (count + 255) / 256 < (1L << 31), "ka_add_scaled: bad count %ld", count);
+    if (count == 0) return 0;
+    hipLaunchKernelGGL(add_scaled_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, x, delta, scale, count);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Two LayerNorms of the same fp32 rows with gains and shifts of their own (a block whose two
+// branches each normalise the block's input), the row read once for both: the mean and variance
+// are the same, only gain and shift differ. Optionally, before that, x += scale * delta, the sum of the
+// branch outputs of the block before, and, whether added or not, delta is cleared for the branches of
+// this block to add into. Without gains (gamma1 null) only that first part runs.
+// ----------------------------------------------------------------------------
+template <typename TOut>
+__global__ void __launch_bounds__(LN_THREADS)
+layernorm_pair_kernel(float* __restrict__ x, float* __restrict__ delta, float scale, int apply,
+                      const float* __restrict__ gamma1, const float* __restrict__ beta1,
+                      const float* __restrict__ gamma2, const float* __restrict__ beta2, float eps,
+                      TOut* __restrict__ out1, TOut* __restrict__ out2, int dim) {
+    __shared__ float smem[LN_THREADS / KA_WAVE];
+    const int i = blockIdx.x;
+    float* row = x + (size_t)i * dim;
+    float* drow = delta ? delta + (size_t)i * dim : nullptr;
+    float s = 0.f;
+    for (int d = threadIdx.x; d < dim; d += LN_THREADS) {
+        float v = row[d];
+        if (drow) {
+            if (apply) {
+                v = fmaf(scale, drow[d], v);
+                row[d] = v;
+            }
+            drow[d] = 0.f;
+        }
+        s += v;
+    }
+    if (!gamma1) return;
+    // (every thread reads back only what it has written itself)
+    const float mean = block_sum_256(s, smem) / (float)dim;
+    float q = 0.f;
+    for (int d = threadIdx.x; d < dim; d += LN_THREADS) {
+        const float c = row[d] - mean;
+        q += c * c;
+    }
+    const float rstd = 1.0f / sqrtf(block_sum_256(q, smem) / (float)dim + eps);
+    TOut* dst1 = out1 + (size_t)i * dim;
+    TOut* dst2 = out2 ? out2 + (size_t)i * dim : nullptr;
+    for (int d = threadIdx.x; d < dim; d += LN_THREADS) {
+        const float c = (row[d] - mean) * rstd;
+        float y = c * gamma1[d];
+        if (beta1) y += beta1[d];
+        dst1[d] = ka_from_float<TOut>(y);
+        if (dst2) {
+            float z = c * gamma2[d];
+            if (beta2) z += beta2[d];
+            dst2[d] = ka_from_float<TOut>(z);
+        }
+    }
+}
+
+KA_API int ka_layernorm_pair(float* x, float* delta, float scale, int apply, const float* gamma1, const float* beta1,
+                             const float* gamma2, const float* beta2, float eps, void* out1, void* out2, int out_dtype,
+                             int n, int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0 && eps >= 0.f, "ka_layernorm_pair: bad sizes n=%d dim=%d", n, dim);
+    KA_CHECK(!apply || delta, "ka_layernorm_pair: nothing to add");
+    KA_CHECK(gamma1 || delta, "ka_layernorm_pair: nothing to do");
+    KA_CHECK(!gamma1 || out1, "ka_layernorm_pair: the first norm has no output");
+    KA_CHECK((out2 != nullptr) == (gamma2 != nullptr), "ka_layernorm_pair: the second norm needs gains and an output");
+    KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_layernorm_pair: unsupported out dtype %d", out_dtype);
+    if (n == 0) return 0;
+    dim3 grid(n), block(LN_THREADS);
+    if (out_dtype == KA_F32)
+        hipLaunchKernelGGL(layernorm_pair_kernel<float>, grid, block, 0, stream, x, delta, scale, apply, gamma1, beta1, gamma2,
+                           beta2, eps, (float*)out1, (float*)out2, dim);
+    else
+        hipLaunchKernelGGL(layernorm_pair_kernel<bf16_t>, grid, block, 0, stream, x, delta, scale, apply, gamma1, beta1, gamma2,
+                           beta2, eps, (bf16_t*)out1, (bf16_t*)out2, dim);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Unit-norm queries and keys + paged cache write, for attention without a rotation whose queries and
+// keys are divided, head by head, by their root mean square (x / sqrt(mean(x^2) + eps), no gain;
+// arithmetic in fp32), and whose values may have another size than its keys.
+//
+// qkv row: [H*hd q | Hkv*hd k | Hkv*hdv v]. q and k are normalised in place (normalise != 0); k and v
+// then go into the cache: keys [pages, Hkv, page_size, hd], values [pages, Hkv, hdv, page_size].
+// slots as for ka_rope_cache. One wave per head at a time.
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+unit_norm_cache_kernel(T* __restrict__ qkv, long row_stride, const int* __restrict__ slots, T* __restrict__ k_cache,
+                       T* __restrict__ v_cache, int H, int Hkv, int hd, int hdv, int page_size, float eps, int normalise) {
+    const int t = blockIdx.x;
+    T* row = qkv + (size_t)t * row_stride;
+    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE, waves = blockDim.x / KA_WAVE;
+    const long slot = slots ? slots[t] : -1;
+    const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
+    for (int h = wave; h < H + Hkv; h += waves) {          // (the same trip count for every lane of a wave)
+        T* p = row + (size_t)h * hd;
+        float rinv = 1.f;
+        if (normalise) {
+            float ss = 0.f;
+            for (int d = lane; d < hd; d += KA_WAVE) {
+                const float v = ka_to_float(p[d]);
+                ss = fmaf(v, v, ss);
+            }
+            rinv = 1.0f / sqrtf(ka_wave_sum(ss) / (float)hd + eps);
+        }
+        const bool key = h >= H;
+        T* kdst = key && slot >= 0 ? k_cache + (((size_t)page * Hkv + (h - H)) * page_size + off) * hd : nullptr;
+        for (int d = lane; d < hd; d += KA_WAVE) {
+            const T y = ka_from_float<T>(ka_to_float(p[d]) * rinv);
+            if (normalise) p[d] = y;
+            if (kdst) kdst[d] = y;
+        }
+    }
+    if (slot < 0) return;
+    const T* vrow = row + (size_t)(H + Hkv) * hd;
+    for (int idx = threadIdx.x; idx < Hkv * hdv; idx += blockDim.x) {
+        const int h = idx / hdv, d = idx % hdv;
+        v_cache[(((size_t)page * Hkv + h) * hdv + d) * page_size + off] = vrow[idx];
+    }
+}
+
+KA_API int ka_unit_norm_cache(void* qkv, int dtype, long row_stride, const int* slots, void* k_cache, void* v_cache,
+                              int n, int H, int Hkv, int hd, int hdv, int page_size, float eps, int normalise,
+                              hipStream_t stream) {
+    KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0 && hdv > 0, "ka_unit_norm_cache: bad sizes");
+    KA_CHECK(row_stride >= (long)(H + Hkv) * hd + (long)Hkv * hdv, "ka_unit_norm_cache: row stride %ld too small", row_stride);
+    KA_CHECK(page_size > 0 && eps >= 0.f, "ka_unit_norm_cache: page size %d, eps %g", page_size, eps);
+    KA_CHECK(slots == nullptr || (k_cache && v_cache), "ka_unit_norm_cache: cache tensors missing");
+    if (n == 0) return 0;
+    dim3 grid(n), block(256);
+    if (dtype == KA_F32)
+        hipLaunchKernelGGL(unit_norm_cache_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, slots,
+                           (float*)k_cache, (float*)v_cache, H, Hkv, hd, hdv, page_size, eps, normalise);
+    else if (dtype == KA_BF16)
+        hipLaunchKernelGGL(unit_norm_cache_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, row_stride, slots,
+                           (bf16_t*)k_cache, (bf16_t*)v_cache, H, Hkv, hd, hdv, page_size, eps, normalise);
+    else
+        KA_CHECK(false, "ka_unit_norm_cache: unsupported dtype %d", dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}

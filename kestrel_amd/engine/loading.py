@@ -33,7 +33,8 @@ def load_model(model_dir, dtype: torch.dtype, device: torch.device, model: Optio
     spec, _typed, plan = read_model_dir(model_dir, model)
     net = DecoderModel(plan)
     tensors = load_tensors(weights_file or find_weights(model_dir, spec.filename), net.params(), dtype, device=device,
-                           prefixes=spec.tensor_prefixes, foreign_prefixes=spec.foreign_prefixes)
+                           prefixes=spec.tensor_prefixes,
+                           foreign_prefixes=tuple(spec.foreign_prefixes) + tuple(getattr(plan, "ignored_prefixes", ())))
     net.bind(tensors, dtype, device)
     return net
 

@@ -35,7 +35,7 @@ def parse_args(argv=None):
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time (each rounded up to 64)")
     parser.add_argument("--page-size", type=int, default=16, help="tokens per cache page (must divide 64)")
-    parser.add_argument("--max-requests", type=int, default=64, help="most requests live at a time")
+    parser.add_argument("--max-requests", type=int, default=4, help="request slots: most requests live at a time")
     parser.add_argument("--device", default="cuda:0")
     return parser.parse_args(argv)
 

@@ -25,7 +25,12 @@ class DecoderModel:
         self.blocks: List[Block] = [Block(layer) for layer in plan.layers]
         self.final_norm = build_part("norm", plan.final_norm)
         self.position = build_part("position", plan.position) if plan.position is not None else None
+        self.junctions = {name: build_part("junction", spec) for name, spec in dict(getattr(plan, "junctions", None) or {}).items()}
         for index, entry in enumerate(plan.schedule):
+            before = getattr(entry, "before", None)
+            if before is not None and before not in self.junctions:
+                raise ValueError(f"schedule entry {index} passes through the junction {before!r}, the plan has "
+                                 f"{sorted(self.junctions) or 'none'}")
             if not 0 <= entry.layer < len(self.blocks):
                 raise ValueError(f"schedule entry {index} names layer {entry.layer}, the plan has {len(self.blocks)}")
             if entry.reads_cache_of is not None:
@@ -51,6 +56,9 @@ class DecoderModel:
         if self.position is not None:
             for local, pspec in self.position.params().items():
                 out[plan.names[f"position.{local}"]] = pspec
+        for name, junction in self.junctions.items():
+            for local, pspec in junction.params().items():
+                out[plan.names[f"junction.{name}.{local}"]] = pspec
         if not plan.tied_head:
             out[plan.names["head.weight"]] = ParamSpec((plan.vocab_size, plan.dim), "matrix", "normal")
         if plan.head_bias:
@@ -67,6 +75,8 @@ class DecoderModel:
                              device)
         if self.position is not None:
             self.position.bind({k: tensors[plan.names[f"position.{k}"]] for k in self.position.params()}, dtype, device)
+        for name, junction in self.junctions.items():
+            junction.bind({k: tensors[plan.names[f"junction.{name}.{k}"]] for k in junction.params()}, dtype, device)
         self.head_weight = self.embedding if plan.tied_head else tensors[plan.names["head.weight"]].to(device).contiguous()
         if plan.head_bias:
             self.head_bias = tensors[plan.names["head.bias"]].to(device=device, dtype=torch.float32).contiguous()
@@ -88,7 +98,7 @@ class DecoderModel:
     def replays_every_step(self) -> bool:
         """Whether steps of every shape may be captured and replayed: every part of the model says so
         (``Part.replays_every_step``)."""
-        parts = [self.final_norm, self.position]
+        parts = [self.final_norm, self.position] + list(self.junctions.values())
         for block in self.blocks:
             parts += list(block.parts().values()) + [getattr(block.mixer, "position", None)]
         return all(bool(getattr(part, "replays_every_step", False)) for part in parts if part is not None)
@@ -117,10 +127,17 @@ class DecoderModel:
             core.scatter_rows(batch.given_embeds, batch.given_rows, x)
         if self.position is not None:
             self.position.add_to_embeddings(x, batch)
+        for junction in self.junctions.values():
+            junction.begin(x, batch)
         handed = None      # the next block's first norm of x, where a block's last launch has computed it
         for index, entry in enumerate(plan.schedule):
             after = plan.schedule[index + 1] if index + 1 < len(plan.schedule) else None
-            then = self.blocks[after.layer].norm if after is not None else None
+            # (a junction between two runs changes the stream: no norm is handed across it)
+            then = self.blocks[after.layer].norm if after is not None and getattr(after, "before", None) is None else None
+            before = getattr(entry, "before", None)
+            if before is not None:
+                self.junctions[before].forward(x, batch)
+                handed = None
             handed = self.blocks[entry.layer].forward(x, batch, caches[index], normed=handed, then=then)
         wanted = int(batch.logit_rows.numel())
         logits = ws.get("model.logits", (wanted, plan.vocab_size), torch.float32)

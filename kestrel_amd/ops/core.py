@@ -31,7 +31,14 @@ _SIGNATURES = {
                           _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                              _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
-                             _c_int, _c_void_p],
+                             _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p],
+    "ka_add_table_rows": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_cast_columns": [_c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],
+    "ka_add_scaled": [_c_void_p, _c_void_p, _c_float, _c_long, _c_void_p],
+    "ka_layernorm_pair": [_c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float,
+                          _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_unit_norm_cache": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                           _c_int, _c_int, _c_float, _c_int, _c_void_p],
     "ka_argmax": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
     "ka_suppress_tokens": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_allow_tokens": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
@@ -110,14 +117,17 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
-def _check_caches(who: str, k_cache, v_cache, dtype, n_kv_heads: int, page_size: int, head_dim: int) -> None:
-    """Keys ``[pages, Hkv, page_size, hd]``, values ``[pages, Hkv, hd, page_size]``, both contiguous."""
+def _check_caches(who: str, k_cache, v_cache, dtype, n_kv_heads: int, page_size: int, head_dim: int,
+                  value_dim: Optional[int] = None) -> None:
+    """Keys ``[pages, Hkv, page_size, hd]``, values ``[pages, Hkv, hdv, page_size]`` (``hdv``: ``value_dim``, the
+    head size unless given), both contiguous."""
+    value_dim = head_dim if value_dim is None else value_dim
     _need(k_cache.dtype == dtype and k_cache.is_contiguous() and k_cache.dim() == 4
           and tuple(k_cache.shape[1:]) == (n_kv_heads, page_size, head_dim),
           f"{who}: key cache must be [pages, Hkv, page_size, hd] of the activation type")
     _need(v_cache.dtype == dtype and v_cache.is_contiguous() and v_cache.dim() == 4
-          and tuple(v_cache.shape[1:]) == (n_kv_heads, head_dim, page_size) and v_cache.shape[0] == k_cache.shape[0],
-          f"{who}: value cache must be [pages, Hkv, hd, page_size] of the activation type")
+          and tuple(v_cache.shape[1:]) == (n_kv_heads, value_dim, page_size) and v_cache.shape[0] == k_cache.shape[0],
+          f"{who}: value cache must be [pages, Hkv, hdv, page_size] of the activation type")
 
 
 def measured_peaks(device: torch.device, read_bytes: int = 2 << 30) -> dict:
@@ -213,6 +223,86 @@ def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
                               code_of(out.dtype), n, dim, stream_ptr()))
 
 
+def add_table_rows(table: torch.Tensor, places: torch.Tensor, x: torch.Tensor) -> None:
+    """``x[t] += table[places[t]]`` in fp32 (learned position vectors; a place outside the table adds nothing)."""
+    _dev(table, places, x)
+    n, dim = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "add_table_rows: x must be contiguous fp32")
+    _need(table.dim() == 2 and table.shape[1] == dim and table.is_contiguous(), "add_table_rows: table must be [rows, dim]")
+    _need(places.dtype == torch.int32 and places.numel() == n and places.is_contiguous(), "add_table_rows: places int32 [n]")
+    _check(lib().ka_add_table_rows(table.data_ptr(), code_of(table.dtype), table.shape[0], places.data_ptr(), x.data_ptr(),
+                                   n, dim, stream_ptr()))
+
+
+def cast_columns(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """``dst[:, :] = src`` for fp32 rows ``src`` and a ``dst`` that may be a range of columns of wider rows
+    (a view with a row stride of its own) of either activation type."""
+    _dev(src, dst)
+    n, dim = src.shape
+    _need(src.dtype == torch.float32 and src.is_contiguous(), "cast_columns: src must be contiguous fp32")
+    _need(dst.dim() == 2 and tuple(dst.shape) == (n, dim) and dst.stride(1) == 1, "cast_columns: dst must be [n, dim] rows")
+    _check(lib().ka_cast_columns(src.data_ptr(), dst.data_ptr(), code_of(dst.dtype), dst.stride(0) if n > 1 else max(dst.stride(0), dim),
+                                 n, dim, stream_ptr()))
+
+
+def add_scaled(x: torch.Tensor, delta: torch.Tensor, scale: float) -> None:
+    """``x += scale * delta`` (both contiguous fp32 of one shape)."""
+    _dev(x, delta)
+    _need(x.dtype == torch.float32 and delta.dtype == torch.float32 and x.is_contiguous() and delta.is_contiguous()
+          and x.shape == delta.shape, "add_scaled: two contiguous fp32 tensors of one shape")
+    _check(lib().ka_add_scaled(x.data_ptr(), delta.data_ptr(), float(scale), x.numel(), stream_ptr()))
+
+
+def layernorm_pair(x: torch.Tensor, first, second, out1: Optional[torch.Tensor], out2: Optional[torch.Tensor],
+                   delta: Optional[torch.Tensor] = None, scale: float = 1.0, apply: bool = False) -> None:
+    """Two LayerNorms of the same fp32 rows in one pass: ``out1 = LN(x; first)`` and, if ``second`` is given,
+    ``out2 = LN(x; second)``, each of ``first`` / ``second`` being ``(gamma, beta or None, eps)`` with one ``eps``.
+    ``delta`` (fp32, the shape of ``x``): cleared, after ``x += scale * delta`` if ``apply``. ``first`` ``None``: only that."""
+    _dev(x, out1, out2, delta)
+    n, dim = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "layernorm_pair: x must be contiguous fp32")
+    _need(delta is None or (delta.dtype == torch.float32 and delta.is_contiguous() and delta.shape == x.shape),
+          "layernorm_pair: delta must be fp32 of the shape of x")
+    g1 = b1 = g2 = b2 = None
+    eps = 0.0
+    if first is not None:
+        g1, b1, eps = first
+        _need(out1 is not None and out1.is_contiguous() and tuple(out1.shape) == (n, dim), "layernorm_pair: out1 must be [n, dim]")
+        if second is not None:
+            g2, b2, eps2 = second
+            _need(float(eps2) == float(eps), "layernorm_pair: the two norms must share eps")
+            _need(out2 is not None and out2.is_contiguous() and tuple(out2.shape) == (n, dim) and out2.dtype == out1.dtype,
+                  "layernorm_pair: out2 must be [n, dim] of out1's type")
+        for t in (g1, b1, g2, b2):
+            _need(t is None or (t.dtype == torch.float32 and t.numel() == dim and t.is_cuda), "layernorm_pair: gains and shifts fp32 [dim]")
+    else:
+        _need(second is None and delta is not None, "layernorm_pair: nothing to do")
+    _check(lib().ka_layernorm_pair(x.data_ptr(), _ptr(delta), float(scale), int(bool(apply)), _ptr(g1), _ptr(b1), _ptr(g2), _ptr(b2),
+                                   float(eps), _ptr(out1) if first is not None else None,
+                                   _ptr(out2) if second is not None else None,
+                                   code_of(out1.dtype) if first is not None else KA_F32, n, dim, stream_ptr()))
+
+
+def unit_norm_cache(qkv: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                    v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
+                    page_size: int, eps: Optional[float]) -> None:
+    """Divide every query and key head of ``qkv`` ``[n, H hd | Hkv hd | Hkv hdv]`` by its root mean square
+    (``x / sqrt(mean(x^2) + eps)``, in place; ``eps`` ``None``: left as they are) and write keys and values into the
+    paged cache (keys ``[pages, Hkv, page_size, hd]``, values ``[pages, Hkv, hdv, page_size]``; ``slots`` ``None``
+    writes nothing)."""
+    _dev(qkv, slots, k_cache, v_cache)
+    n = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim,
+          "unit_norm_cache: qkv must be [n, H hd + Hkv hd + Hkv hdv]")
+    if slots is not None:
+        _need(slots.dtype == torch.int32 and slots.numel() == n and slots.is_contiguous(), "unit_norm_cache: slots int32 [n]")
+        _need(k_cache is not None and v_cache is not None, "unit_norm_cache: cache tensors missing")
+        _check_caches("unit_norm_cache", k_cache, v_cache, qkv.dtype, n_kv_heads, page_size, head_dim, value_dim)
+    _check(lib().ka_unit_norm_cache(qkv.data_ptr(), code_of(qkv.dtype), qkv.stride(0) if n > 1 else qkv.shape[1], _ptr(slots),
+                                    _ptr(k_cache), _ptr(v_cache), n, n_heads, n_kv_heads, head_dim, value_dim, page_size,
+                                    float(eps or 0.0), int(eps is not None), stream_ptr()))
+
+
 ROTARY_PAIRINGS = {"halves": 0, "interleaved": 1}
 
 
@@ -269,15 +359,28 @@ def linear_generic(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
 
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       token_row: torch.Tensor, kv_lo: Optional[torch.Tensor], kv_hi: torch.Tensor,
-                      out: torch.Tensor, scale: float, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
-    """Paged attention of ``n`` packed tokens; ``q`` may be a strided view into a qkv buffer."""
-    _dev(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out)
+                      out: torch.Tensor, scale: float, n_heads: int, n_kv_heads: int, head_dim: int,
+                      value_dim: Optional[int] = None, positions: Optional[torch.Tensor] = None,
+                      slopes: Optional[torch.Tensor] = None, sink: Optional[float] = None) -> None:
+    """Paged attention of ``n`` packed tokens; ``q`` may be a strided view into a qkv buffer.
+
+    ``value_dim``: size of a value head where it differs from ``head_dim`` (``out`` is ``[n, H value_dim]``).
+    ``slopes`` (fp32 ``[H]``) with ``positions`` (int32 ``[n]``): the score of a query at place ``i`` against the key
+    at place ``j`` is lowered by ``slopes[h] * (i - j)``. ``sink``: the score of one more term of the softmax's
+    denominator that carries no value (``None``: no such term)."""
+    _dev(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, positions, slopes)
     n = q.shape[0]
+    value_dim = head_dim if value_dim is None else int(value_dim)
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * head_dim, "attention: q must be [n, >= H hd]")
-    _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * head_dim) and out.dtype == q.dtype,
-          "attention: out must be [n, H hd] of the q type")
+    _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * value_dim) and out.dtype == q.dtype,
+          "attention: out must be [n, H hdv] of the q type")
     page_size = k_cache.shape[2]
-    _check_caches("attention", k_cache, v_cache, q.dtype, n_kv_heads, page_size, head_dim)
+    _check_caches("attention", k_cache, v_cache, q.dtype, n_kv_heads, page_size, head_dim, value_dim)
+    if slopes is not None:
+        _need(slopes.dtype == torch.float32 and slopes.numel() == n_heads and slopes.is_contiguous(),
+              "attention: slopes must be fp32 [H]")
+        _need(positions is not None and positions.dtype == torch.int32 and positions.numel() == n and positions.is_contiguous(),
+              "attention: slopes need the queries' positions, int32 [n]")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "attention: block table must be contiguous int32 [rows, pages]")
     for t in (token_row, kv_hi) + ((kv_lo,) if kv_lo is not None else ()):
@@ -286,7 +389,8 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                                       v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
                                       token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
                                       out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size,
-                                      stream_ptr()))
+                                      value_dim, _ptr(positions) if slopes is not None else None, _ptr(slopes),
+                                      int(sink is not None), float(sink or 0.0), stream_ptr()))
 
 
 def _pending_args(who: str, rows: int, pending, pending_at):

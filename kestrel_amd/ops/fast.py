@@ -578,3 +578,15 @@ def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, ou
             int(batch.max_kv) if batch.max_kv > 1 else 0, size, stream_ptr()))
         return True
     return False
+
+
+def biased_query_block(head_dim: int, value_dim: int) -> Optional[int]:
+    """Queries of one row that a workgroup of the MFMA kernel for attention with distance slopes, a sink and values of
+    a size of their own takes, or ``None`` where that kernel does not cover the sizes."""
+    return None
+
+
+def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
+                          head_dim, value_dim, positions, slopes, sink, batch) -> bool:
+    """Attention with the further terms of ``ops.core.attention_generic`` on the matrix cores. False: not covered."""
+    return False

@@ -28,6 +28,15 @@ class PagedAttention(Mixer):
     and the pairing of channels); ``None`` means q and k go into attention as they are. Nothing
     else is understood here: an encoding that needs more (several axes, a learned table added to
     the input) is refused when the weights are bound, not silently turned the rotary way.
+
+    Further forms, each switched on by its field of the specification and all of them together or alone:
+    values of another size than keys (``value_dim``: the cache's value pages and the output projection follow);
+    queries and keys divided head by head by their root mean square before the scores (``qk_unit_norm_eps``);
+    scores lowered by a head's slope times the distance ``i - j`` between query and key (``distance_slopes``);
+    a term in the softmax's denominator that has a score but no value (``sink``), so that a query may attend to
+    nothing; the three projections stored as three tensors (``split_projections``). With any of the middle four
+    the mixer takes no rotation, and runs through kernels of its own (``ops.core.unit_norm_cache`` and the
+    attention kernels that know these terms).
     """
 
     replays_every_step = True
@@ -38,9 +47,19 @@ class PagedAttention(Mixer):
             raise ValueError(f"{spec.n_heads} query heads cannot share {spec.n_kv_heads} kv heads")
         self.position = build_part("position", spec.position)
         self.scale = float(spec.scale) if spec.scale is not None else float(spec.head_dim) ** -0.5
+        self.value_dim = int(spec.head_dim if getattr(spec, "value_dim", None) is None else spec.value_dim)
         self.q_dim = spec.n_heads * spec.head_dim
         self.kv_dim = spec.n_kv_heads * spec.head_dim
-        self.qkv_dim = self.q_dim + 2 * self.kv_dim
+        self.v_dim = spec.n_kv_heads * self.value_dim
+        self.qkv_dim = self.q_dim + self.kv_dim + self.v_dim
+        self.out_dim = spec.n_heads * self.value_dim
+        self.unit_norm_eps = getattr(spec, "qk_unit_norm_eps", None)
+        self.sink = getattr(spec, "sink", None)
+        self.distance = getattr(spec, "distance_slopes", None)
+        # the forms that the kernels of the rotary path know nothing of
+        self.extended = self.value_dim != spec.head_dim or self.unit_norm_eps is not None or self.sink is not None \
+            or self.distance is not None
+        self._slopes: Optional[torch.Tensor] = None
         self.qkv_weight = self.qkv_bias = self.proj_weight = self.proj_bias = None
         self.dtype: Optional[torch.dtype] = None
         self._table = None
@@ -48,23 +67,37 @@ class PagedAttention(Mixer):
 
     def params(self) -> Dict[str, ParamSpec]:
         spec = self.spec
-        out = {"qkv.weight": ParamSpec((self.qkv_dim, spec.dim)), "proj.weight": ParamSpec((spec.dim, self.q_dim))}
+        pieces = {"q": self.q_dim, "k": self.kv_dim, "v": self.v_dim} if getattr(spec, "split_projections", False) \
+            else {"qkv": self.qkv_dim}
+        out = {f"{name}.weight": ParamSpec((rows, spec.dim)) for name, rows in pieces.items()}
+        out["proj.weight"] = ParamSpec((spec.dim, self.out_dim))
         if spec.bias:
-            out["qkv.bias"] = ParamSpec((self.qkv_dim,), "vector", "bias")
+            out.update({f"{name}.bias": ParamSpec((rows,), "vector", "bias") for name, rows in pieces.items()})
             out["proj.bias"] = ParamSpec((spec.dim,), "vector", "bias")
         return out
 
     def cache_spec(self) -> CacheSpec:
-        return CacheSpec(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
+        return CacheSpec(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window,
+                         self.value_dim if self.value_dim != self.spec.head_dim else None)
 
     def bind(self, tensors, dtype, device) -> None:
         spec = self.spec
         self.dtype = dtype
-        self.qkv_weight = tensors["qkv.weight"].to(device).contiguous()
+        split = getattr(spec, "split_projections", False)
+
+        def fused(what: str) -> torch.Tensor:
+            # (rows of q, then k, then v: the order of a fused projection's outputs)
+            if split:
+                return torch.cat([tensors[f"{name}.{what}"].to(device) for name in ("q", "k", "v")], dim=0)
+            return tensors[f"qkv.{what}"].to(device)
+
+        self.qkv_weight = fused("weight").contiguous()
         self.proj_weight = tensors["proj.weight"].to(device).contiguous()
         if self.spec.bias:
-            self.qkv_bias = tensors["qkv.bias"].to(device=device, dtype=torch.float32).contiguous()
+            self.qkv_bias = fused("bias").to(dtype=torch.float32).contiguous()
             self.proj_bias = tensors["proj.bias"].to(device=device, dtype=torch.float32).contiguous()
+        if self.distance is not None:
+            self._slopes = torch.tensor(self.distance.values(spec.n_heads), dtype=torch.float32, device=device)
         if int(getattr(self.position, "axes", 1)) != 1:
             raise ValueError(f"attention rotates by a token's place in the sequence; the position encoding "
                              f"{getattr(spec.position, 'kind', '?')!r} takes {self.position.axes} numbers per token")
@@ -80,6 +113,9 @@ class PagedAttention(Mixer):
             if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] % 2 or table.shape[1] > self.spec.head_dim:
                 raise ValueError(f"a rotation's table must be fp32 [positions, R] with R even and at most the head size "
                                  f"{self.spec.head_dim}, got {tuple(table.shape)} {table.dtype}")
+            if self.extended:
+                raise ValueError("attention with values of another size, unit-norm queries and keys, distance slopes or a "
+                                 "sink takes no rotation")
             self._table, self._pairing = table.to(device).contiguous(), rotation.pairing
         else:
             self._table, self._pairing = None, "halves"
@@ -88,6 +124,8 @@ class PagedAttention(Mixer):
         if self.dtype != torch.bfloat16:
             return None                     # the generic kernel takes tokens one by one
         from ..ops import fast
+        if self.extended:
+            return fast.biased_query_block(self.spec.head_dim, self.value_dim)
         return fast.prefill_query_block(self.spec.head_dim)
 
     # The three stages are also offered one by one, so that a block may fuse the first with its
@@ -101,7 +139,7 @@ class PagedAttention(Mixer):
     def _decodes_fused(self, batch, cache: LayerCache) -> bool:
         """One token per row in bf16 with a rotation by halves: the decode kernel then rotates q and
         k and stores k and v itself."""
-        return self.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None \
+        return self.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None and not self.extended \
             and self._pairing == "halves"          # the MFMA-path kernels turn halves; the generic one any pairing
 
     def takes_beside(self, job, batch, cache: LayerCache) -> bool:
@@ -116,7 +154,11 @@ class PagedAttention(Mixer):
         spec = self.spec
         n = qkv.shape[0]
         group = batch.groups[cache.group]
-        out = batch.workspace.get("attn.out", (n, self.q_dim), self.dtype)
+        out = batch.workspace.get("attn.out", (n, self.out_dim), self.dtype)
+        if self.extended:
+            if beside is not None:
+                self._alone(beside)
+            return self._attend_extended(qkv, batch, cache, group, out)
         halves = self._pairing == "halves"
         if qkv.dtype == torch.bfloat16 and self._decodes_fused(batch, cache):
             from ..ops import fast
@@ -146,6 +188,23 @@ class PagedAttention(Mixer):
                             spec.head_dim, group.page_size, self._pairing)
         paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                         self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
+        return out
+
+    def _attend_extended(self, qkv, batch, cache: LayerCache, group, out):
+        """Queries and keys to unit norm, the cache write, then attention with the terms the specification names."""
+        spec = self.spec
+        slots = group.slots if cache.writes else None
+        core.unit_norm_cache(qkv, slots, cache.k, cache.v, spec.n_heads, spec.n_kv_heads, spec.head_dim, self.value_dim,
+                             group.page_size, self.unit_norm_eps)
+        if qkv.dtype == torch.bfloat16:
+            from ..ops import fast
+            if fast.attention_biased_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi,
+                                          out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, self.value_dim,
+                                          batch.positions, self._slopes, self.sink, batch):
+                return out
+        core.attention_generic(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
+                               self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, self.value_dim, batch.positions,
+                               self._slopes, self.sink)
         return out
 
     @staticmethod

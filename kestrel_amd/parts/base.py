@@ -5,7 +5,7 @@ A part is built from its specification alone, says which tensors it owns
 (``forward``). It never sees the model or the architecture it is used in.
 
 Adding a part of a new kind: subclass the interface, and call ``register_mixer`` /
-``register_feed_forward`` / ``register_norm`` / ``register_position`` with the kind
+``register_feed_forward`` / ``register_norm`` / ``register_position`` / ``register_junction`` with the kind
 name that its specification carries.
 """
 
@@ -90,6 +90,20 @@ class PositionEncoding(Part):
         """Model-level encodings: add the encoding of every token's position into the fp32 rows ``x``
         ``[tokens, dim]`` in place (``batch.positions``, ``batch.position_axes``). Under replayed graphs
         (``batch.decode_only``) this must neither synchronise nor allocate."""
+
+
+class Junction(Part):
+    """A transformation of the whole residual stream between two runs of layers (``ScheduleEntry.before``).
+
+    ``begin`` is called once a step with the embedding output (after the model's position encoding), before the
+    first run; ``forward`` replaces fp32 ``x`` in place at every place of the schedule that names the junction.
+    Both must keep the promises of ``Part`` under replayed graphs."""
+
+    def begin(self, x: torch.Tensor, batch) -> None:
+        """See the embedding output ``x`` ``[tokens, dim]`` of this step."""
+
+    def forward(self, x: torch.Tensor, batch) -> None:
+        raise NotImplementedError
 
 
 @dataclass
@@ -190,7 +204,7 @@ class FeedForward(Part):
         return None
 
 
-_REGISTRIES: Dict[str, Dict[str, Callable]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}}
+_REGISTRIES: Dict[str, Dict[str, Callable]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "junction": {}}
 
 
 def _register(family: str, kind: str, cls: Callable) -> None:
@@ -211,6 +225,10 @@ def register_norm(kind: str, cls: Callable) -> None:
 
 def register_position(kind: str, cls: Callable) -> None:
     _register("position", kind, cls)
+
+
+def register_junction(kind: str, cls: Callable) -> None:
+    _register("junction", kind, cls)
 
 
 def build_part(family: str, spec) -> Part:

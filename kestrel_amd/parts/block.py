@@ -103,7 +103,36 @@ def _sequential(block: "Block", x, batch, cache) -> None:
     block.feed_forward.forward(h, batch, x)
 
 
-ARRANGEMENTS: Dict[str, Callable] = {"parallel": _parallel, "sequential": _sequential}
+def _parallel_two_norms(block: "Block", x, batch, cache) -> None:
+    """``x + residual_scale * (mixer(norm(x)) + ff(norm2(x)))``: two branches, each with a norm of its own of the
+    same ``x``; without a feed-forward, ``x + residual_scale * mixer(norm(x))``.
+
+    Both norms come from one pass over ``x`` where they are LayerNorms of one eps. The branches add into a
+    buffer of their own, which enters the stream with the weight (in fp32, like the stream)."""
+    from ..ops import core
+
+    ws = batch.workspace
+    h1 = ws.get("block.h", tuple(x.shape), block.dtype)
+    delta = ws.get("block.delta", tuple(x.shape), torch.float32)
+    ff = block.feed_forward
+    ln1 = block.norm.layernorm_operands()
+    ln2 = block.norm2.layernorm_operands() if ff is not None else None
+    h2 = ws.get("block.h2", tuple(x.shape), block.dtype) if ff is not None else None
+    if ln1 is not None and (ff is None or (ln2 is not None and float(ln2[2]) == float(ln1[2]))):
+        core.layernorm_pair(x, ln1, ln2, h1, h2, delta=delta)
+    else:
+        core.layernorm_pair(x, None, None, None, None, delta=delta)
+        block.norm.forward(x, h1)
+        if ff is not None:
+            block.norm2.forward(x, h2)
+    block.mixer.forward(h1, batch, cache, delta)
+    if ff is not None:
+        ff.forward(h2, batch, delta)
+    core.add_scaled(x, delta, block.spec.residual_scale)
+
+
+ARRANGEMENTS: Dict[str, Callable] = {"parallel": _parallel, "sequential": _sequential,
+                                     "parallel_two_norms": _parallel_two_norms}
 
 
 def register_arrangement(name: str, fn: Callable) -> None:
@@ -127,12 +156,18 @@ class Block:
         if spec.arrangement == "sequential" and self.norm2 is None:
             raise ValueError("the sequential arrangement needs norm2")
         self.mixer = build_part("mixer", spec.mixer)
-        self.feed_forward = build_part("feed_forward", spec.feed_forward)
+        if spec.feed_forward is None and spec.arrangement != "parallel_two_norms":
+            raise ValueError(f"the {spec.arrangement} arrangement needs a feed-forward")
+        if spec.arrangement == "parallel_two_norms" and spec.feed_forward is not None and self.norm2 is None:
+            raise ValueError("the parallel_two_norms arrangement needs norm2 for its feed-forward")
+        self.feed_forward = build_part("feed_forward", spec.feed_forward) if spec.feed_forward is not None else None
         self.dtype: Optional[torch.dtype] = None
         self._run = ARRANGEMENTS[spec.arrangement]
 
     def parts(self) -> Dict[str, Part]:
-        out = {"norm": self.norm, "mixer": self.mixer, "feed_forward": self.feed_forward}
+        out = {"norm": self.norm, "mixer": self.mixer}
+        if self.feed_forward is not None:
+            out["feed_forward"] = self.feed_forward
         if self.norm2 is not None:
             out["norm2"] = self.norm2
         return out

@@ -48,6 +48,36 @@ class PositionSpec:
 
 
 @dataclass(frozen=True)
+class LearnedPositionSpec:
+    """One learned vector per position, added to the embedded tokens before the first block."""
+
+    kind: str
+    dim: int
+    max_positions: int
+
+
+@dataclass(frozen=True)
+class ConcatLinearSpec:
+    """A junction of the stack: the residual stream is replaced by one linear of the stream and the
+    embedding output side by side, ``x <- W [x; x0]`` with ``W`` ``[dim, 2 dim]`` (the stream's columns first)."""
+
+    kind: str
+    dim: int
+
+
+@dataclass(frozen=True)
+class DistanceSlopes:
+    """A bias on attention scores that grows with distance: the score of a query at place ``i`` against a key at
+    place ``j`` is lowered by ``slope_h * (i - j)``, with ``slope_h = 2 ** (-exponent * (h + 1) / H)`` for query
+    head ``h`` of ``H``."""
+
+    exponent: float = 8.0
+
+    def values(self, n_heads: int):
+        return [2.0 ** (-self.exponent * (h + 1) / n_heads) for h in range(n_heads)]
+
+
+@dataclass(frozen=True)
 class CacheSpec:
     """What an attention mixer keeps per token: keys and values of ``n_kv_heads`` x ``head_dim``.
 
@@ -65,15 +95,18 @@ class CacheSpec:
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None     # size of a value head where it is not the keys' (``None``: ``head_dim``)
 
     def page_tensors(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
         # values are kept transposed inside a page: eight consecutive keys of one channel are 16
         # bytes, which is what the MFMA attention kernels load at a time
-        return {"k": (self.n_kv_heads, page_size, self.head_dim), "v": (self.n_kv_heads, self.head_dim, page_size)}
+        value_dim = self.head_dim if self.value_dim is None else self.value_dim
+        return {"k": (self.n_kv_heads, page_size, self.head_dim), "v": (self.n_kv_heads, value_dim, page_size)}
 
     @property
     def group_key(self) -> Tuple:
-        return ("kv", self.n_kv_heads, self.head_dim, self.window)
+        value_dim = self.head_dim if self.value_dim is None else self.value_dim
+        return ("kv", self.n_kv_heads, self.head_dim, self.window) + ((value_dim,) if value_dim != self.head_dim else ())
 
 
 @dataclass(frozen=True)
@@ -95,6 +128,17 @@ class AttentionSpec:
     bias: bool = True
     scale: Optional[float] = None  # None: head_dim ** -0.5
     window: Optional[int] = None
+    # size of a value head (``None``: ``head_dim``); the output projection then reads ``n_heads * value_dim`` columns
+    value_dim: Optional[int] = None
+    # the projections of queries, keys and values as three tensors (``q.weight``, ``k.weight``, ``v.weight``) instead of
+    # one (``qkv.weight``); they are laid side by side when the weights are bound
+    split_projections: bool = False
+    # queries and keys divided, head by head, by their root mean square ``sqrt(mean(x^2) + eps)`` (no gain): its eps
+    qk_unit_norm_eps: Optional[float] = None
+    # scores lowered by a head's slope times the distance between query and key
+    distance_slopes: Optional[DistanceSlopes] = None
+    # one more term ``exp(sink)`` in the softmax's denominator that carries no value (``None``: none)
+    sink: Optional[float] = None
 
 
 @dataclass(frozen=True)
@@ -111,7 +155,9 @@ class LayerSpec:
     """One block: its parts, how they are arranged, and where their tensors are named.
 
     ``arrangement``: ``parallel`` = ``x + mixer(norm(x)) + ff(norm(x))`` (one norm);
-    ``sequential`` = ``x += mixer(norm(x)); x += ff(norm2(x))``.
+    ``sequential`` = ``x += mixer(norm(x)); x += ff(norm2(x))``;
+    ``parallel_two_norms`` = ``x + residual_scale * (mixer(norm(x)) + ff(norm2(x)))``, both norms of the same ``x``
+    (``feed_forward`` and ``norm2`` may be ``None`` there: a layer of a mixer alone).
     ``names`` maps ``"<part>.<local tensor name>"`` (parts: ``norm``, ``norm2``, ``mixer``,
     ``feed_forward``) to the tensor's name in the checkpoint.
     """
@@ -122,15 +168,18 @@ class LayerSpec:
     feed_forward: object
     norm2: Optional[object] = None
     names: Mapping[str, str] = field(default_factory=dict)
+    residual_scale: float = 1.0        # weight of the branches' sum in arrangements that have one
 
 
 @dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a layer. ``reads_cache_of``: index of an earlier schedule entry whose
-    cache this run reads instead of keeping one of its own."""
+    cache this run reads instead of keeping one of its own. ``before``: name of a junction of the
+    plan (``ModelPlan.junctions``) that the residual stream passes through right before this run."""
 
     layer: int
     reads_cache_of: Optional[int] = None
+    before: Optional[str] = None
 
 
 @dataclass(frozen=True)
@@ -158,6 +207,12 @@ class ModelPlan:
     # encoding): its ``add_to_embeddings`` runs on the embedded tokens before the first block; its tensors
     # are named by ``names["position.<local name>"]``. ``None``: positions are the mixers' business.
     position: Optional[object] = None
+    # junctions by name: specifications whose parts (registered as junctions) transform the residual stream between
+    # runs of layers, where a schedule entry names one (``ScheduleEntry.before``); a junction named by several
+    # entries runs with the same tensors each time; its tensors are named by ``names["junction.<name>.<local name>"]``
+    junctions: Mapping[str, object] = field(default_factory=dict)
+    # tensors of a checkpoint with these prefixes are passed over (parts that a configuration leaves out)
+    ignored_prefixes: Tuple[str, ...] = ()
 
     def describe(self) -> Dict[str, object]:
         return {"architecture": self.architecture, "layers": len(self.layers), "schedule": len(self.schedule),
