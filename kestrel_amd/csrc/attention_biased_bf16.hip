@@ -1,0 +1,344 @@
+// bf16 paged attention on the matrix cores for mixers whose scores carry a distance bias, whose
+// softmax may have a term without a value (a sink), and whose values may have another size than
+// their keys. One kernel serves prompts, portions, mixed steps and decode steps.
+//
+// Cache layout as everywhere in this folder: keys [pages, Hkv, 16, hd], values [pages, Hkv, hdv, 16]
+// (transposed inside the page), page size 16. Token t of the packed batch reads the keys
+// [kv_lo[t], kv_hi[t]) of its row; the step's own keys are already in the cache, and queries and
+// keys come normalised where the mixer normalises them.
+//
+// The score of query t (place p = positions[t]) of head h against the key at place j is
+//     scale * (q . k) - slopes[h] * (p - j)          (slopes optional)
+// and the weights are exp(s_j) / (sum_j exp(s_j) [+ exp(sink)]): fp32 throughout; the weights enter
+// the value product as bf16, sums in fp32.
+//
+// A workgroup owns 32 columns of the score product and one kv head. In a step with prompt portions a
+// column is a query of a block of 32 consecutive tokens of one row and one query head (the host lists the
+// blocks); in a decode step, where every row has one token, the columns are the query heads that share the
+// kv head (up to 32), so that the row's keys and values are read once for all of them. Its waves take the
+// tiles of 32 keys (two pages) in turn. Scores are computed transposed, S^T = K Q^T, with
+// v_mfma_f32_32x32x16_bf16: a lane then holds 16 scores of ONE column, so the softmax is in-lane work
+// plus one exchange with the lane 32 away. The key rows are fed to the product with bits 2 and 3 of the row index
+// swapped: the 8 weights a lane holds per page are then those of 8 consecutive keys, which is, as they stand,
+// the column operand of O^T += V^T P^T, whose row operand is one 16-byte load from the transposed value
+// page. The outputs are rescaled only when some column's maximum has grown by more than 2^8. Waves merge
+// through LDS in a tree.
+#include "ka_common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 ab_bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 ab_bf16x4;
+typedef __attribute__((ext_vector_type(16))) float ab_floatx16;
+
+constexpr int AB_PAGE = 16;
+constexpr int AB_TILE = 32;                 // keys per tile: two pages
+constexpr int AB_COLS = 32;                 // columns (queries) per workgroup
+constexpr float AB_SLACK = 8.0f;            // powers of two a maximum may grow before the outputs are rescaled
+constexpr float AB_LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ float ab_max_halves(float x) {
+    typedef __attribute__((ext_vector_type(2))) unsigned ab_u2;
+    const ab_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float ab_sum_halves(float x) {
+    typedef __attribute__((ext_vector_type(2))) unsigned ab_u2;
+    const ab_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// NK: 16-channel steps of a query/key head (hd = 16 NK); NV: 32-channel blocks of a value head (hdv <= 32 NV).
+// heads_per_block: 1 = the columns are consecutive tokens of a block of queries (qblk_row / qblk_tok list the blocks,
+// grid (H, blocks)); > 1 = a decode step, the columns are that many query heads of one kv head of token blockIdx.y
+// (grid (Hkv * ceil(G / heads_per_block), tokens)).
+template <int NK, int NV>
+__global__ void __launch_bounds__(512)
+attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
+                   const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
+                   const int* __restrict__ qblk_row, const int* __restrict__ qblk_tok, const int* __restrict__ cu_q,
+                   const int* __restrict__ token_row, const int* __restrict__ kv_lo, const int* __restrict__ kv_hi,
+                   const int* __restrict__ positions, const float* __restrict__ slopes, bf16_t* __restrict__ out,
+                   long out_row_stride, float scale, int H, int Hkv, int hdv, int heads_per_block, int has_sink,
+                   float sink_score) {
+    constexpr int HD = NK * 16;
+    constexpr int REC = 16 * NV + 2;            // floats a lane hands over at a merge: its outputs, m and l
+    extern __shared__ float mrg[];              // [waves / 2][REC][64]
+    const int n_waves = blockDim.x / KA_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KA_WAVE), lane = threadIdx.x % KA_WAVE;
+    const int col = lane % 32, half = lane / 32;
+    const int G = H / Hkv;
+    int kvh, head, tok, row;
+    bool live;
+    if (heads_per_block > 1) {
+        const int groups = (G + heads_per_block - 1) / heads_per_block;
+        kvh = blockIdx.x / groups;
+        const int hq = (blockIdx.x % groups) * heads_per_block + col;
+        live = col < heads_per_block && hq < G;
+        head = kvh * G + (live ? hq : 0);
+        tok = blockIdx.y;
+        row = token_row[tok];
+    } else {
+        head = blockIdx.x;
+        kvh = head / G;
+        const int blk = blockIdx.y;
+        row = qblk_row[blk];
+        const int tok_end = cu_q[row + 1];
+        if (qblk_tok[blk] >= tok_end) return;          // (the unused end of a list of fixed length)
+        tok = qblk_tok[blk] + col;
+        live = tok < tok_end;
+        if (!live) tok = tok_end - 1;
+    }
+    const int hi = live ? kv_hi[tok] : 0;
+    const int lo = live ? (kv_lo ? kv_lo[tok] : 0) : 0;
+    // the block's range of keys, and the part of it that every live column sees whole
+    int blk_hi = ka_lanes_reduce<1, KA_WAVE>(hi, KaIntMax{});
+    int blk_lo = ka_lanes_reduce<1, KA_WAVE>(live && hi > lo ? lo : 0x7fffffff, KaIntMin{});
+    int min_hi = ka_lanes_reduce<1, KA_WAVE>(live ? hi : 0x7fffffff, KaIntMin{});
+    int max_lo = ka_lanes_reduce<1, KA_WAVE>(live ? lo : 0, KaIntMax{});
+    blk_hi = __builtin_amdgcn_readfirstlane(blk_hi);
+    blk_lo = __builtin_amdgcn_readfirstlane(blk_lo);
+    min_hi = __builtin_amdgcn_readfirstlane(min_hi);
+    max_lo = __builtin_amdgcn_readfirstlane(max_lo);
+
+    // queries: the column operand of the score product, held for the whole loop
+    ab_bf16x8 qreg[NK];
+    {
+        const bf16_t* qp = q + (size_t)tok * q_row_stride + (size_t)head * HD + half * 8;
+#pragma unroll
+        for (int c = 0; c < NK; ++c) qreg[c] = *reinterpret_cast<const ab_bf16x8*>(qp + c * 16);
+    }
+    const float slope2 = slopes ? slopes[head] * AB_LOG2E : 0.f;     // in powers of two, like everything below
+    const float scale2 = scale * AB_LOG2E;
+    const int place = slopes ? positions[tok] : 0;
+    const float sink2 = sink_score * AB_LOG2E;
+
+    float m = has_sink ? sink2 : -INFINITY;     // reference point of this lane's column (the same in both halves)
+    float l = 0.f;                              // this lane's share of the column's sum
+    ab_floatx16 o[NV];
+#pragma unroll
+    for (int b = 0; b < NV; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[b][i] = 0.f;
+
+    const int* table = block_table + (size_t)row * max_pages;
+    // the key this lane loads for the score product: row `col` of the product is key perm(col) of the tile
+    const int krow = (col & 0x13) | ((col & 4) << 1) | ((col & 8) >> 1);
+    const int kpage_in_tile = krow >> 4, kslot = krow & 15;
+    const size_t k_head = (size_t)kvh * AB_PAGE * HD, k_page = (size_t)Hkv * AB_PAGE * HD;
+    const size_t v_page = (size_t)Hkv * hdv * AB_PAGE;
+    // the value rows (channels) this lane loads: clamped into the head where the last block is not full
+    int vch[NV];
+#pragma unroll
+    for (int b = 0; b < NV; ++b) vch[b] = min(b * 32 + col, hdv - 1);
+
+    if (blk_lo < blk_hi) {
+        const int first_tile = blk_lo / AB_TILE, last_tile = (blk_hi - 1) / AB_TILE;
+        for (int tile = first_tile + wave; tile <= last_tile; tile += n_waves) {
+            const int base = tile * AB_TILE;
+            // pages of the tile (a page the row has given back, or none: any page, its keys are masked)
+            int pg[2];
+#pragma unroll
+            for (int p = 0; p < 2; ++p) {
+                const int e = table[min(tile * 2 + p, max_pages - 1)];
+                pg[p] = e < 0 ? 0 : e;
+            }
+            ab_bf16x8 kr[NK];
+            {
+                const bf16_t* kp = k_cache + (size_t)pg[kpage_in_tile] * k_page + k_head + (size_t)kslot * HD + half * 8;
+#pragma unroll
+                for (int c = 0; c < NK; ++c) kr[c] = *reinterpret_cast<const ab_bf16x8*>(kp + c * 16);
+            }
+            ab_bf16x8 vr[2][NV];
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+#pragma unroll
+                for (int b = 0; b < NV; ++b)
+                    vr[p][b] = *reinterpret_cast<const ab_bf16x8*>(v_cache + (size_t)pg[p] * v_page +
+                                                                   ((size_t)kvh * hdv + vch[b]) * AB_PAGE + half * 8);
+            ab_floatx16 s;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[i] = 0.f;
+#pragma unroll
+            for (int c = 0; c < NK; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[c], qreg[c], s, 0, 0, 0);
+            // register i of this lane: key base + (i / 8) * 16 + half * 8 + i % 8 of the lane's column
+            const int j0 = base + half * 8;
+            const float bias0 = -slope2 * (float)(place - j0);          // (an integer distance: exact)
+            const bool whole = base >= max_lo && base + AB_TILE <= min_hi;
+            if (!whole) {
+                // Keys that no column of the block sees (slots behind the row's last key, pages given back) may hold
+                // anything, a NaN included, and a weight of 0 does not clear that in a product: their values are zeroed.
+#pragma unroll
+                for (int p = 0; p < 2; ++p)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int j = base + p * AB_PAGE + half * 8 + e;
+                        if (j < blk_lo || j >= blk_hi) {
+#pragma unroll
+                            for (int b = 0; b < NV; ++b) vr[p][b][e] = (bf16_t)0.f;
+                        }
+                    }
+            }
+            float tile_max = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int off = (i / 8) * 16 + i % 8;
+                float x = fmaf(s[i], scale2, fmaf(slope2, (float)off, bias0));
+                if (!whole) {
+                    const int j = j0 + off;
+                    if (j < lo || j >= hi) x = -INFINITY;
+                }
+                s[i] = x;
+                tile_max = fmaxf(tile_max, x);
+            }
+            tile_max = ab_max_halves(tile_max);
+            // the reference point moves only when some column's maximum has outgrown it by 2^slack
+            if (__builtin_amdgcn_ballot_w64(tile_max > m + AB_SLACK) != 0) {
+                const float m_new = fmaxf(m, tile_max);
+                const float corr = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+                l *= corr;
+#pragma unroll
+                for (int b = 0; b < NV; ++b)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o[b][i] *= corr;
+                m = m_new;
+            }
+            const float ref = m == -INFINITY ? 0.f : m;
+            ab_bf16x8 pb[2];
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float p = __builtin_amdgcn_exp2f(s[i] - ref);      // (a masked key: exp2(-inf) = 0)
+                sum += p;
+                pb[i / 8][i % 8] = (bf16_t)p;
+            }
+            l += sum;
+#pragma unroll
+            for (int p = 0; p < 2; ++p)
+#pragma unroll
+                for (int b = 0; b < NV; ++b) o[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vr[p][b], pb[p], o[b], 0, 0, 0);
+        }
+    }
+    l = ab_sum_halves(l);                       // the column's whole sum, in both of its lanes
+
+    // merge the waves in a tree: in round r the waves with bit r set hand over to the wave 2^r below
+    for (int step = 1; step < n_waves; step <<= 1) {
+        const bool gives = (wave & (2 * step - 1)) == step, takes = (wave & (2 * step - 1)) == 0 && wave + step < n_waves;
+        float* slot = mrg + (size_t)(wave / (2 * step)) * REC * KA_WAVE;
+        if (gives) {
+#pragma unroll
+            for (int b = 0; b < NV; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) slot[(b * 16 + i) * KA_WAVE + lane] = o[b][i];
+            slot[(16 * NV) * KA_WAVE + lane] = m;
+            slot[(16 * NV + 1) * KA_WAVE + lane] = l;
+        }
+        __syncthreads();
+        if (takes) {
+            const float m2 = slot[(16 * NV) * KA_WAVE + lane], l2 = slot[(16 * NV + 1) * KA_WAVE + lane];
+            const float m_new = fmaxf(m, m2);
+            const float c1 = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+            const float c2 = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m2 - m_new);
+#pragma unroll
+            for (int b = 0; b < NV; ++b)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[b][i] = o[b][i] * c1 + slot[(b * 16 + i) * KA_WAVE + lane] * c2;
+            l = l * c1 + l2 * c2;
+            m = m_new;
+        }
+        __syncthreads();
+    }
+    if (wave != 0 || !live) return;
+    if (has_sink) {
+        const float m_new = fmaxf(m, sink2);
+        const float c = __builtin_amdgcn_exp2f(m - m_new);
+        l = l * c + __builtin_amdgcn_exp2f(sink2 - m_new);
+#pragma unroll
+        for (int b = 0; b < NV; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[b][i] *= c;
+    }
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
+    // register i of block b: channel b * 32 + (i / 4) * 8 + half * 4 + i % 4 of the lane's column
+    bf16_t* op = out + (size_t)tok * out_row_stride + (size_t)head * hdv;
+#pragma unroll
+    for (int b = 0; b < NV; ++b)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+            const int ch = b * 32 + g4 * 8 + half * 4;
+            if (ch + 3 < hdv) {
+                ab_bf16x4 y;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) y[e] = (bf16_t)(o[b][g4 * 4 + e] * inv);
+                *reinterpret_cast<ab_bf16x4*>(op + ch) = y;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (ch + e < hdv) op[ch + e] = (bf16_t)(o[b][g4 * 4 + e] * inv);
+            }
+        }
+}
+
+static bool ab_sizes_covered(int hd, int hdv) {
+    const int nk = hd / 16, nv = (hdv + 31) / 32;
+    return hd % 16 == 0 && hdv % 4 == 0 && (nk == 2 || nk == 3 || nk == 4 || nk == 6 || nk == 8) && nv >= 1 && nv <= 4;
+}
+
+// Whether the kernel covers these sizes: query/key heads of 32, 48, 64, 96 or 128 channels, value heads of up to
+// 128 in steps of 4, pages of 16.
+KA_API int ka_attention_biased_supported(int hd, int hdv, int page_size) {
+    return page_size == AB_PAGE && ab_sizes_covered(hd, hdv) ? 1 : 0;
+}
+
+KA_API int ka_attention_biased_query_block() { return AB_COLS; }
+
+// n_blocks > 0: a step with blocks of queries (qblk_row, qblk_tok; cu_q); n_blocks == 0: a decode step of n tokens,
+// one per row. waves: 4 or 8 per workgroup.
+KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
+                                    const int* block_table, int max_pages, const int* qblk_row, const int* qblk_tok,
+                                    int n_blocks, const int* cu_q, const int* token_row, const int* kv_lo,
+                                    const int* kv_hi, const int* positions, const float* slopes, void* out,
+                                    long out_row_stride, float scale, int n, int H, int Hkv, int hd, int hdv,
+                                    int page_size, int waves, int has_sink, float sink_score, hipStream_t stream) {
+    const char* who = "ka_attention_biased_bf16";
+    KA_CHECK(n >= 0 && n_blocks >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes", who);
+    KA_CHECK(page_size == AB_PAGE && ab_sizes_covered(hd, hdv), "%s: head sizes %d / %d or page size %d not covered", who, hd, hdv, page_size);
+    KA_CHECK(max_pages > 0, "%s: bad table width %d", who, max_pages);
+    KA_CHECK(waves == 4 || waves == 8, "%s: %d waves", who, waves);
+    KA_CHECK((uintptr_t)q % 16 == 0 && q_row_stride % 8 == 0 && (uintptr_t)k_cache % 16 == 0 && (uintptr_t)v_cache % 16 == 0,
+             "%s: operands must be 16-byte aligned", who);
+    KA_CHECK((uintptr_t)out % 8 == 0 && out_row_stride % 4 == 0, "%s: output rows must be 8-byte aligned", who);
+    KA_CHECK(slopes == nullptr || positions != nullptr, "%s: slopes need the queries' positions", who);
+    KA_CHECK(n_blocks == 0 || (qblk_row && qblk_tok && cu_q), "%s: blocks of queries need their lists", who);
+    if (n == 0) return 0;
+    const int G = H / Hkv;
+    int heads_per_block = 1;
+    dim3 grid;
+    if (n_blocks > 0) {
+        grid = dim3(H, n_blocks);
+    } else {
+        // (with a single query head per kv head the columns hold one query: heads_per_block 1 would mean blocks)
+        heads_per_block = G < 2 ? 2 : (G > AB_COLS ? AB_COLS : G);
+        grid = dim3(Hkv * ((G + heads_per_block - 1) / heads_per_block), n);
+        KA_CHECK(n <= 65535, "%s: too many decode rows %d", who, n);
+    }
+    KA_CHECK(grid.y <= 65535, "%s: too many blocks %d", who, (int)grid.y);
+    const int nk = hd / 16, nv = (hdv + 31) / 32;
+    const size_t lds = (size_t)(waves / 2) * (16 * nv + 2) * KA_WAVE * sizeof(float);
+#define AB_LAUNCH(NK, NV)                                                                                                  \
+    if (nk == NK && nv == NV) {                                                                                            \
+        static bool sized = false;                                                                                         \
+        if (!sized) {                                                                                                      \
+            (void)hipFuncSetAttribute((const void*)attn_biased_kernel<NK, NV>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            sized = true;                                                                                                  \
+        }                                                                                                                  \
+        hipLaunchKernelGGL((attn_biased_kernel<NK, NV>), grid, dim3(KA_WAVE * waves), lds, stream, (const bf16_t*)q,       \
+                           q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, \
+                           qblk_tok, cu_q, token_row, kv_lo, kv_hi, positions, slopes, (bf16_t*)out, out_row_stride, scale, \
+                           H, Hkv, hdv, heads_per_block, has_sink, sink_score);                                            \
+    }
+#define AB_LAUNCH_NK(NK) AB_LAUNCH(NK, 1) AB_LAUNCH(NK, 2) AB_LAUNCH(NK, 3) AB_LAUNCH(NK, 4)
+    AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(6) AB_LAUNCH_NK(8)
+#undef AB_LAUNCH_NK
+#undef AB_LAUNCH
+    KA_LAUNCH_CHECK();
+    return 0;
+}

@@ -52,6 +52,9 @@ _SIGNATURES = {
         _c_void_p, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,          # the tokens' own keys and values
         _c_void_p, _c_long, _c_int,                                                                  # A, lda, K
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],      # W, ldw, bias, out, ..., stream
+    "ka_attention_biased_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
+                                 _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p],
     "ka_linear_skinny_norm_store": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p,
                                     _c_int, _c_long, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
 }
@@ -150,6 +153,10 @@ def lib():
         for name in ("ka_attention_prefill_supported", "ka_attention_decode_supported"):
             getattr(handle, name).argtypes = [_c_int, _c_int]
             getattr(handle, name).restype = _c_int
+        handle.ka_attention_biased_supported.argtypes = [_c_int] * 3
+        handle.ka_attention_biased_supported.restype = _c_int
+        handle.ka_attention_biased_query_block.argtypes = []
+        handle.ka_attention_biased_query_block.restype = _c_int
         handle.ka_attention_decode_beside_supported.argtypes = [_c_int] * 6
         handle.ka_attention_decode_beside_supported.restype = _c_int
         for name in ("ka_attention_prefill_max_keys", "ka_attention_prefill_query_block"):
@@ -583,10 +590,51 @@ def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, ou
 def biased_query_block(head_dim: int, value_dim: int) -> Optional[int]:
     """Queries of one row that a workgroup of the MFMA kernel for attention with distance slopes, a sink and values of
     a size of their own takes, or ``None`` where that kernel does not cover the sizes."""
-    return None
+    handle = lib()
+    if not handle.ka_attention_biased_supported(int(head_dim), int(value_dim), 16):
+        return None
+    return int(handle.ka_attention_biased_query_block())
 
 
 def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
                           head_dim, value_dim, positions, slopes, sink, batch) -> bool:
-    """Attention with the further terms of ``ops.core.attention_generic`` on the matrix cores. False: not covered."""
-    return False
+    """Attention with the further terms of ``ops.core.attention_generic`` (values of ``value_dim`` channels, ``slopes``
+    times the distance taken off the scores, a ``sink`` in the softmax's denominator) on the matrix cores, for prompt
+    portions, mixed steps and decode steps alike. False: not covered (head sizes, page size, alignment, no list of
+    blocks of 32 queries with the step), nothing was run."""
+    n = q.shape[0]
+    page_size = k_cache.shape[2]
+    if n == 0:
+        return True
+    handle = lib()
+    if batch is None or not handle.ka_attention_biased_supported(int(head_dim), int(value_dim), int(page_size)):
+        return False
+    if q.dtype != torch.bfloat16 or q.data_ptr() % 16 or q.stride(0) % 8 or q.stride(1) != 1 or out.data_ptr() % 8 \
+            or out.stride(0) % 4 or out.stride(1) != 1 or k_cache.data_ptr() % 16 or v_cache.data_ptr() % 16:
+        return False
+    if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or positions is None):
+        raise KernelError("attention: slopes must be fp32 [H] and come with the queries' positions")
+    if batch.decode_only:
+        rows = first = None
+        n_blocks = 0
+        groups = n_heads // n_kv_heads
+        workgroups = n * n_kv_heads * -(-groups // 32)
+        waves = 4 if workgroups >= 2 * chip_sizes(q.device).compute_units else 8
+    else:
+        size = int(handle.ka_attention_biased_query_block())
+        listed = (getattr(batch, "query_blocks", None) or {}).get(size)
+        if listed is None:
+            return False
+        rows, first = listed
+        n_blocks = int(rows.numel())
+        if n_blocks == 0 or n_blocks > 65535:
+            return False
+        waves = 4
+    if n > 65535:
+        return False
+    _check(handle.ka_attention_biased_bf16(
+        q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+        _ptr(rows), _ptr(first), n_blocks, batch.cu_q.data_ptr(), token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(),
+        _ptr(positions), _ptr(slopes), out.data_ptr(), out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim,
+        value_dim, page_size, waves, int(sink is not None), float(sink or 0.0), stream_ptr()))
+    return True
