@@ -14,6 +14,10 @@ the whole engine instead: a model folder is written with seeded random weights, 
 loader, and requests go through ``InferenceEngine`` (scheduler, sampler, paged cache under
 pressure); the line then reports generated tokens a second. With ``--check N`` (meant for ``--layers 2``) the first N
 greedy requests of such a run are compared, token by token, with the plain implementation under ``tests/``.
+
+``--workload compare-vimesun`` measures the Vimesun design beside the Moondream decoder at equal sizes (width,
+feed-forward, heads, head size, runs of layers, vocabulary; random weights): a prompt alone and decode steps at batch 1,
+8 and 64 through the same step function, each with its share of the roofline (``--compare-sizes``, ``--compare-model``).
 """
 
 from __future__ import annotations
@@ -63,6 +67,126 @@ def build_model(layers: int, dtype, device, sizes=None):
                for name, pspec in net.params().items()}
     net.bind(tensors, dtype, device)
     return net, typed
+
+
+def build_from_config(config: dict, model: str, dtype, device):
+    """A model of any registered architecture from its ``config.json`` dictionary, random weights drawn on the GPU."""
+    import torch
+
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.weights import InitRecipe, random_tensor
+
+    spec = get_spec(model)
+    typed = spec.read_config(config)
+    net = DecoderModel(spec.build_plan(typed))
+    recipe = InitRecipe(std=0.02)
+    tensors = {name: random_tensor(name, pspec, SEED, recipe, device=device).to(torch.bfloat16 if dtype == torch.bfloat16 else dtype)
+               for name, pspec in net.params().items()}
+    net.bind(tensors, dtype, device)
+    return net, typed
+
+
+# Sizes at which the two designs are measured side by side: (label, width, feed-forward, heads, kv heads, head size,
+# value head size of Vimesun, window of Vimesun or None for its position limit, layers, looped stretch and passes).
+# Moondream gets as many layers as Vimesun has runs of layers; its values have the keys' size.
+COMPARE_SIZES = {
+    "w2048": dict(width=2048, ff=8192, heads=32, kv_heads=32, head=64, vdim=64, window=None, layers=4, loop=(1, 3, 2)),
+    "w2048-window": dict(width=2048, ff=8192, heads=32, kv_heads=32, head=64, vdim=64, window=512, layers=4, loop=(1, 3, 2)),
+    "w4096-gqa": dict(width=4096, ff=11008, heads=32, kv_heads=8, head=128, vdim=128, window=None, layers=3, loop=(1, 2, 2)),
+    "w2560-v": dict(width=2560, ff=10240, heads=32, kv_heads=8, head=64, vdim=96, window=1024, layers=4, loop=(1, 3, 2)),
+}
+COMPARE_VOCAB = 51200
+
+
+def compare_models(size: dict, positions: int):
+    """``{name: (config dict, registry name, facts)}`` of the two designs at one size; ``facts`` is what the roofline
+    needs: runs of layers, and per run the linears' weights and the attention's sizes."""
+    from types import SimpleNamespace
+
+    start, stop, times = size["loop"]
+    runs = size["layers"] + (stop - start) * (times - 1)
+    mixer = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["head"], "vdim": size["vdim"],
+             "scale": size["head"] ** -0.5}
+    if size["window"]:
+        mixer["mask"] = {"size": size["window"]}
+    else:
+        mixer["mask"] = {"size": positions}
+    vimesun = {"architecture": "Vimesun", "vocab": COMPARE_VOCAB, "width": size["width"], "max_positions": positions,
+               "norm": {"eps": 1e-5}, "residual_mult": 0.7, "loop": dict(zip(("start", "stop", "times"), size["loop"])),
+               "layers": [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": size["ff"]}}
+                          for _ in range(size["layers"])]}
+    moondream = {"text": {"dim": size["width"], "ff_dim": size["ff"], "n_layers": runs, "vocab_size": COMPARE_VOCAB,
+                          "max_context": positions, "n_heads": size["heads"], "n_kv_heads": size["kv_heads"],
+                          "head_dim": size["head"], "rotary_dim": size["head"] // 2, "rope_theta": 10000.0,
+                          "prefix_attn": 0, "layer_norm_eps": 1e-5}}
+    w, h, g, d = size["width"], size["heads"], size["kv_heads"], size["head"]
+
+    def facts(dv, window, junctions):
+        linear = w * (h * d + g * d + g * dv) + h * dv * w + 2 * w * size["ff"]        # weights of one run's linears
+        return SimpleNamespace(runs=runs, linear=linear, extra=junctions * 2 * w * w, heads=h, kv_heads=g, d=d, dv=dv,
+                               window=window, width=w, vocab=COMPARE_VOCAB)
+
+    return {"vimesun": (vimesun, "vimesun", facts(size["vdim"], size["window"], times)),
+            "moondream2": (moondream, "moondream2", facts(d, None, 0))}
+
+
+def compare_flops(f, tokens: int) -> float:
+    """Multiply-adds x 2 of a prompt of ``tokens`` places: linears, score and value products over the keys each
+    place sees, the head at the last place."""
+    seen = sum(min(p + 1, f.window or p + 1) for p in range(tokens))
+    return 2.0 * tokens * (f.runs * f.linear + f.extra) + 2.0 * f.runs * f.heads * (f.d + f.dv) * seen + 2.0 * f.width * f.vocab
+
+
+def compare_decode_bytes(f, batch: int, context: int, size: int) -> float:
+    """Bytes a decode step must read: every weight once, and of every row the keys and values it sees."""
+    keys = min(context, f.window or context)
+    return size * (f.runs * f.linear + f.extra + f.width * f.vocab + batch * f.runs * f.kv_heads * (f.d + f.dv) * keys)
+
+
+def run_compare(args, dtype, device) -> dict:
+    """Vimesun beside the Moondream decoder at equal sizes, through the same step function."""
+    from types import SimpleNamespace
+
+    import torch
+
+    size_bytes = 2 if dtype == torch.bfloat16 else 4
+    context, tokens = args.context, args.prefill_tokens
+    positions = max(context + args.steps + args.warmup + 16, tokens)
+    out = {}
+    for label in args.compare_sizes.split(","):
+        size = COMPARE_SIZES[label]
+        out[label] = {}
+        for name, (config, registry_name, f) in compare_models(size, positions).items():
+            if args.compare_model not in ("both", name):
+                continue
+            net, _typed = build_from_config(config, registry_name, dtype, device)
+            # (what the timing harness asks of a typed configuration)
+            shim = SimpleNamespace(prefix_attn=0, dim=f.width, vocab_size=f.vocab, n_kv_heads=f.kv_heads,
+                                   head_dim=(f.d + f.dv) / 2, n_layers=f.runs)
+            entry = {}
+            seconds, best = time_prefill(net, shim, tokens, repeats=5)
+            flops = compare_flops(f, tokens)
+            entry["prefill"] = {"tokens": tokens, "ms": round(seconds * 1e3, 3), "best_ms": round(best * 1e3, 3),
+                                "tok_s": round(tokens / seconds, 1), "frac_of_peak_flops": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+            for batch in (1, 8, 64):
+                steps = args.steps if batch < 64 else max(16, args.steps // 4)
+                elapsed, _kv = time_decode(net, shim, batch, context, steps, min(args.warmup, 4))
+                moved = compare_decode_bytes(f, batch, context, size_bytes)
+                entry[f"decode_b{batch}"] = {"ms_per_step": round(elapsed / steps * 1e3, 4), "tok_s": round(batch * steps / elapsed, 1),
+                                             "frac_of_peak_hbm": round(moved / (elapsed / steps) / PEAK_HBM, 4)}
+            out[label][name] = entry
+            del net
+            torch.cuda.empty_cache()
+    first = out[args.compare_sizes.split(",")[0]]
+    lead = first.get("vimesun") or next(iter(first.values()))
+    return {"metric": f"Vimesun beside the Moondream decoder at equal sizes: decode tok/s at batch 8, context {context} ({args.compare_sizes.split(',')[0]})",
+            "value": lead["decode_b8"]["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": lead["decode_b8"]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": args.dtype, "data": "synthetic (seeded random token ids, random weights N(0,0.02))",
+            "config": {"model": "vimesun and moondream2-text at equal sizes", "sizes": {k: COMPARE_SIZES[k] for k in out},
+                       "global_batch": 8, "seq_len": context, "vocab_size": COMPARE_VOCAB, "parallelism": "single-gpu"},
+            "compare": out}
 
 
 def model_bytes(net, dtype_size: int) -> int:
@@ -352,8 +476,13 @@ def main() -> int:
                         help="with --workload: RuntimeConfig.tune_linears (time the vendor library's algorithms at warm-up)")
     parser.add_argument("--check", type=int, default=0,
                         help="with --workload: compare this many greedy requests with the plain implementation (for --layers 2)")
-    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48"],
-                        help="decode: the benchmark's decode step (default); the others run requests through InferenceEngine")
+    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun"],
+                        help="decode: the benchmark's decode step (default); waves256 and mixed48 run requests through "
+                             "InferenceEngine; compare-vimesun measures the Vimesun design beside the Moondream decoder at equal sizes")
+    parser.add_argument("--compare-sizes", default="w2048,w2048-window,w4096-gqa,w2560-v",
+                        help="with --workload compare-vimesun: which of the sizes, with commas between them")
+    parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "moondream2"],
+                        help="with --workload compare-vimesun: one of the two designs only (for profiling)")
     parser.add_argument("--max-batch-size", type=int, default=None, help="for the workloads through the entry point")
     parser.add_argument("--linears", default="library", choices=["library", "own"],
                         help="linears of more than 64 rows (a prompt's): through hipBLASLt (the engine's default) or "
@@ -379,6 +508,9 @@ def main() -> int:
     sizes["max_context"] = max(sizes["max_context"], args.context + max(args.steps, 16) + args.warmup + 8, args.prefill_tokens)
     if args.layers is None:
         args.layers = sizes["n_layers"]
+    if args.workload == "compare-vimesun":
+        print(json.dumps(run_compare(args, dtype, device)))
+        return 0
     if args.workload != "decode":
         print(json.dumps(run_workload(args, dict(SIZES[args.sizes]))))
         return 0

@@ -15,7 +15,7 @@ import torch
 from ..ops import core
 from ..ops.linear import linear
 from ..parts.base import LayerCache, build_part
-from ..parts.block import Block
+from ..parts.block import Block, settle
 from ..parts.specs import ModelPlan, ParamSpec
 
 
@@ -136,9 +136,11 @@ class DecoderModel:
             then = self.blocks[after.layer].norm if after is not None and getattr(after, "before", None) is None else None
             before = getattr(entry, "before", None)
             if before is not None:
+                settle(x, batch)
                 self.junctions[before].forward(x, batch)
                 handed = None
             handed = self.blocks[entry.layer].forward(x, batch, caches[index], normed=handed, then=then)
+        settle(x, batch)       # (what the last block has left to be added into the stream)
         wanted = int(batch.logit_rows.numel())
         logits = ws.get("model.logits", (wanted, plan.vocab_size), torch.float32)
         if wanted:

@@ -103,12 +103,57 @@ def _sequential(block: "Block", x, batch, cache) -> None:
     block.feed_forward.forward(h, batch, x)
 
 
+# Whether a block of weighted branches leaves the sum ``x += scale * delta`` to whoever reads the stream next (the
+# next such block adds it in the pass that computes its norms; anything else calls ``settle`` first) instead of
+# adding it in a launch of its own. Off: every block leaves the stream complete (what a test that reads the
+# stream between blocks needs).
+DEFER_RESIDUAL = True
+_PENDING = "residual_pending"
+
+
+def settle(x, batch) -> None:
+    """Add what a block before has left to be added into the fp32 stream ``x``."""
+    from ..ops import core
+
+    host = getattr(batch, "host", None)
+    pending = host.pop(_PENDING, None) if host else None
+    if pending is not None:
+        core.add_scaled(x, pending[0], pending[1])
+
+
+def _two_branches_few_rows(block: "Block", h1, h2, batch, cache, delta) -> bool:
+    """Both branches for a few bf16 rows: the two first linears, the mixer's core, and both last linears adding into
+    ``delta`` in one launch. Needs a mixer and a feed-forward that offer their stages; ``False`` otherwise."""
+    from ..ops import fast
+    from ..ops.linear import linear
+
+    n = h1.shape[0]
+    ff = block.feed_forward
+    if ff is None or block.dtype != torch.bfloat16 or n > fast.SKINNY_MAX_ROWS:
+        return False
+    m_in, f_in = block.mixer.input_projection(), ff.input_projection()
+    m_out, f_out = block.mixer.output_projection(), ff.output_projection()
+    if m_in is None or f_in is None or m_out is None or f_out is None:
+        return False
+    ws = batch.workspace
+    projected = ws.get("block.mixer_in", (n, m_in[2]), block.dtype)
+    hidden = ws.get("block.ff_hidden", (n, f_in[2]), block.dtype)
+    linear(h1, m_in[0], m_in[1], projected)
+    linear(h2, f_in[0], f_in[1], hidden, act=f_in[3])
+    mixed = block.mixer.attend(projected, batch, cache)
+    if not fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], delta):
+        linear(mixed, m_out[0], m_out[1], delta, accumulate=True)
+        linear(hidden, f_out[0], f_out[1], delta, accumulate=True)
+    return True
+
+
 def _parallel_two_norms(block: "Block", x, batch, cache) -> None:
     """``x + residual_scale * (mixer(norm(x)) + ff(norm2(x)))``: two branches, each with a norm of its own of the
     same ``x``; without a feed-forward, ``x + residual_scale * mixer(norm(x))``.
 
-    Both norms come from one pass over ``x`` where they are LayerNorms of one eps. The branches add into a
-    buffer of their own, which enters the stream with the weight (in fp32, like the stream)."""
+    Both norms come from one pass over ``x`` where they are LayerNorms of one eps; that pass also adds what the
+    block before has left to be added (``DEFER_RESIDUAL``) and clears the buffer the branches add into. The
+    branches' sum enters the stream with the weight in fp32, like the stream."""
     from ..ops import core
 
     ws = batch.workspace
@@ -118,17 +163,29 @@ def _parallel_two_norms(block: "Block", x, batch, cache) -> None:
     ln1 = block.norm.layernorm_operands()
     ln2 = block.norm2.layernorm_operands() if ff is not None else None
     h2 = ws.get("block.h2", tuple(x.shape), block.dtype) if ff is not None else None
+    pending = batch.host.get(_PENDING)
+    if pending is not None and pending[0].data_ptr() != delta.data_ptr():
+        settle(x, batch)              # (left in another buffer than this block's)
+        pending = None
     if ln1 is not None and (ff is None or (ln2 is not None and float(ln2[2]) == float(ln1[2]))):
-        core.layernorm_pair(x, ln1, ln2, h1, h2, delta=delta)
+        core.layernorm_pair(x, ln1, ln2, h1, h2, delta=delta, scale=pending[1] if pending else 1.0, apply=pending is not None)
     else:
-        core.layernorm_pair(x, None, None, None, None, delta=delta)
+        core.layernorm_pair(x, None, None, None, None, delta=delta, scale=pending[1] if pending else 1.0, apply=pending is not None)
         block.norm.forward(x, h1)
         if ff is not None:
             block.norm2.forward(x, h2)
-    block.mixer.forward(h1, batch, cache, delta)
-    if ff is not None:
-        ff.forward(h2, batch, delta)
-    core.add_scaled(x, delta, block.spec.residual_scale)
+    batch.host.pop(_PENDING, None)
+    if not _two_branches_few_rows(block, h1, h2, batch, cache, delta):
+        block.mixer.forward(h1, batch, cache, delta)
+        if ff is not None:
+            ff.forward(h2, batch, delta)
+    if DEFER_RESIDUAL:
+        batch.host[_PENDING] = (delta, float(block.spec.residual_scale))
+    else:
+        core.add_scaled(x, delta, block.spec.residual_scale)
+
+
+_parallel_two_norms.defers = True
 
 
 ARRANGEMENTS: Dict[str, Callable] = {"parallel": _parallel, "sequential": _sequential,
@@ -194,6 +251,8 @@ class Block:
         """Updates the fp32 residual ``x`` in place. ``normed``: this block's first norm of ``x``, if the
         block before has computed it; ``then``: the first norm of the block that follows. Returns that
         norm of the result where the block's last launch computed it, else ``None``."""
+        if not getattr(self._run, "defers", False):
+            settle(x, batch)          # (an arrangement that knows nothing of sums left to be added)
         if getattr(self._run, "hands_over", False):
             return self._run(self, x, batch, cache, normed=normed, then=then)
         self._run(self, x, batch, cache)
