@@ -396,7 +396,7 @@ KA_API int ka_add_scaled(float* x, const float* delta, float scale, long count, 
 // ----------------------------------------------------------------------------
 template <typename TOut>
 __global__ void __launch_bounds__(LN_THREADS)
-layernorm_pair_kernel(float* __restrict__ x, float* __restrict__ delta, float scale, int apply,
+layernorm_pair_kernel(float* __restrict__ x, float* __restrict__ delta, float scale, int apply, int clear,
                       const float* __restrict__ gamma1, const float* __restrict__ beta1,
                       const float* __restrict__ gamma2, const float* __restrict__ beta2, float eps,
                       TOut* __restrict__ out1, TOut* __restrict__ out2, int dim) {
@@ -412,7 +412,7 @@ layernorm_pair_kernel(float* __restrict__ x, float* __restrict__ delta, float sc
                 v = fmaf(scale, drow[d], v);
                 row[d] = v;
             }
-            drow[d] = 0.f;
+            if (clear) drow[d] = 0.f;
         }
         s += v;
     }
@@ -440,23 +440,114 @@ layernorm_pair_kernel(float* __restrict__ x, float* __restrict__ delta, float sc
     }
 }
 
-KA_API int ka_layernorm_pair(float* x, float* delta, float scale, int apply, const float* gamma1, const float* beta1,
-                             const float* gamma2, const float* beta2, float eps, void* out1, void* out2, int out_dtype,
-                             int n, int dim, hipStream_t stream) {
+// The same for rows of up to 256 * 4 * ITEMS values that are 16-byte aligned: every thread keeps its share of the
+// row in registers, so the row (and what is added to it) is read once.
+template <typename TOut, int ITEMS>
+__global__ void __launch_bounds__(LN_THREADS)
+layernorm_pair_regs_kernel(float* __restrict__ x, float* __restrict__ delta, float scale, int apply, int clear,
+                           const float* __restrict__ gamma1, const float* __restrict__ beta1,
+                           const float* __restrict__ gamma2, const float* __restrict__ beta2, float eps,
+                           TOut* __restrict__ out1, TOut* __restrict__ out2, int dim) {
+    typedef __attribute__((ext_vector_type(4))) float floatx4;
+    typedef TOut __attribute__((ext_vector_type(4))) out4;
+    __shared__ float smem[LN_THREADS / KA_WAVE];
+    const int i = blockIdx.x;
+    float* row = x + (size_t)i * dim;
+    float* drow = delta ? delta + (size_t)i * dim : nullptr;
+    floatx4 v[ITEMS];
+    float s = 0.f;
+    // (loads first, all of them in flight together; then the arithmetic and the stores)
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int d = min((j * LN_THREADS + (int)threadIdx.x) * 4, dim - 4);
+        v[j] = *reinterpret_cast<const floatx4*>(row + d);
+    }
+    if (drow && apply) {
+        floatx4 a[ITEMS];
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int d = min((j * LN_THREADS + (int)threadIdx.x) * 4, dim - 4);
+            a[j] = *reinterpret_cast<const floatx4*>(drow + d);
+        }
+#pragma unroll
+        for (int j = 0; j < ITEMS; ++j) {
+            const int d = (j * LN_THREADS + threadIdx.x) * 4;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[j][e] = fmaf(scale, a[j][e], v[j][e]);
+            if (d < dim) *reinterpret_cast<floatx4*>(row + d) = v[j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int d = (j * LN_THREADS + threadIdx.x) * 4;
+        if (d >= dim) v[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        else if (drow && clear) *reinterpret_cast<floatx4*>(drow + d) = floatx4{0.f, 0.f, 0.f, 0.f};
+        s += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
+    }
+    if (!gamma1) return;
+    const float mean = block_sum_256(s, smem) / (float)dim;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int d = (j * LN_THREADS + threadIdx.x) * 4;
+        if (d < dim) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) q += (v[j][e] - mean) * (v[j][e] - mean);
+        }
+    }
+    const float rstd = 1.0f / sqrtf(block_sum_256(q, smem) / (float)dim + eps);
+    TOut* dst1 = out1 + (size_t)i * dim;
+    TOut* dst2 = out2 ? out2 + (size_t)i * dim : nullptr;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        const int d = (j * LN_THREADS + threadIdx.x) * 4;
+        if (d < dim) {
+            const floatx4 g1 = *reinterpret_cast<const floatx4*>(gamma1 + d);
+            const floatx4 b1 = beta1 ? *reinterpret_cast<const floatx4*>(beta1 + d) : floatx4{0.f, 0.f, 0.f, 0.f};
+            out4 y;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) y[e] = ka_from_float<TOut>((v[j][e] - mean) * rstd * g1[e] + b1[e]);
+            *reinterpret_cast<out4*>(dst1 + d) = y;
+            if (dst2) {
+                const floatx4 g2 = *reinterpret_cast<const floatx4*>(gamma2 + d);
+                const floatx4 b2 = beta2 ? *reinterpret_cast<const floatx4*>(beta2 + d) : floatx4{0.f, 0.f, 0.f, 0.f};
+                out4 z;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) z[e] = ka_from_float<TOut>((v[j][e] - mean) * rstd * g2[e] + b2[e]);
+                *reinterpret_cast<out4*>(dst2 + d) = z;
+            }
+        }
+    }
+}
+
+// clear: delta is zeroed (after it was added, if apply), for branches that add into it.
+KA_API int ka_layernorm_pair(float* x, float* delta, float scale, int apply, int clear, const float* gamma1,
+                             const float* beta1, const float* gamma2, const float* beta2, float eps, void* out1, void* out2,
+                             int out_dtype, int n, int dim, hipStream_t stream) {
     KA_CHECK(n >= 0 && dim > 0 && eps >= 0.f, "ka_layernorm_pair: bad sizes n=%d dim=%d", n, dim);
-    KA_CHECK(!apply || delta, "ka_layernorm_pair: nothing to add");
-    KA_CHECK(gamma1 || delta, "ka_layernorm_pair: nothing to do");
+    KA_CHECK((!apply && !clear) || delta, "ka_layernorm_pair: nothing to add or clear");
+    KA_CHECK(gamma1 || (delta && (apply || clear)), "ka_layernorm_pair: nothing to do");
     KA_CHECK(!gamma1 || out1, "ka_layernorm_pair: the first norm has no output");
     KA_CHECK((out2 != nullptr) == (gamma2 != nullptr), "ka_layernorm_pair: the second norm needs gains and an output");
     KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_layernorm_pair: unsupported out dtype %d", out_dtype);
     if (n == 0) return 0;
     dim3 grid(n), block(LN_THREADS);
-    if (out_dtype == KA_F32)
-        hipLaunchKernelGGL(layernorm_pair_kernel<float>, grid, block, 0, stream, x, delta, scale, apply, gamma1, beta1, gamma2,
-                           beta2, eps, (float*)out1, (float*)out2, dim);
-    else
-        hipLaunchKernelGGL(layernorm_pair_kernel<bf16_t>, grid, block, 0, stream, x, delta, scale, apply, gamma1, beta1, gamma2,
-                           beta2, eps, (bf16_t*)out1, (bf16_t*)out2, dim);
+    auto aligned = [](const void* p) { return p == nullptr || (uintptr_t)p % 16 == 0; };
+    const bool regs = dim % 4 == 0 && dim <= LN_THREADS * 4 * 4 && aligned(x) && aligned(delta) && aligned(gamma1) && aligned(beta1) &&
+                      aligned(gamma2) && aligned(beta2) && aligned(out1) && aligned(out2);
+#define KA_LNP(KERNEL, TOUT)                                                                                              \
+    hipLaunchKernelGGL((KERNEL), grid, block, 0, stream, x, delta, scale, apply, clear, gamma1, beta1, gamma2, beta2, eps, \
+                       (TOUT*)out1, (TOUT*)out2, dim)
+#define KA_LNP_REGS(ITEMS)                                                        \
+    if (out_dtype == KA_F32) { KA_LNP((layernorm_pair_regs_kernel<float, ITEMS>), float); } \
+    else { KA_LNP((layernorm_pair_regs_kernel<bf16_t, ITEMS>), bf16_t); }
+    if (regs && dim <= LN_THREADS * 4) { KA_LNP_REGS(1) }
+    else if (regs && dim <= LN_THREADS * 4 * 2) { KA_LNP_REGS(2) }
+    else if (regs) { KA_LNP_REGS(4) }
+    else if (out_dtype == KA_F32) { KA_LNP(layernorm_pair_kernel<float>, float); }
+    else { KA_LNP(layernorm_pair_kernel<bf16_t>, bf16_t); }
+#undef KA_LNP_REGS
+#undef KA_LNP
     KA_LAUNCH_CHECK();
     return 0;
 }
@@ -468,41 +559,56 @@ KA_API int ka_layernorm_pair(float* x, float* delta, float scale, int apply, con
 //
 // qkv row: [H*hd q | Hkv*hd k | Hkv*hdv v]. q and k are normalised in place (normalise != 0); k and v
 // then go into the cache: keys [pages, Hkv, page_size, hd], values [pages, Hkv, hdv, page_size].
-// slots as for ka_rope_cache. One wave per head at a time.
+// slots as for ka_rope_cache. A wave per head of a token, four heads a workgroup.
 // ----------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256)
 unit_norm_cache_kernel(T* __restrict__ qkv, long row_stride, const int* __restrict__ slots, T* __restrict__ k_cache,
                        T* __restrict__ v_cache, int H, int Hkv, int hd, int hdv, int page_size, float eps, int normalise) {
+    // a wave per head of a token: the query heads, then the key heads, then the value heads
     const int t = blockIdx.x;
+    const int lane = threadIdx.x % KA_WAVE;
+    const int h = blockIdx.y * (blockDim.x / KA_WAVE) + threadIdx.x / KA_WAVE;
+    if (h >= H + 2 * Hkv) return;
     T* row = qkv + (size_t)t * row_stride;
-    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE, waves = blockDim.x / KA_WAVE;
     const long slot = slots ? slots[t] : -1;
     const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
-    for (int h = wave; h < H + Hkv; h += waves) {          // (the same trip count for every lane of a wave)
-        T* p = row + (size_t)h * hd;
-        float rinv = 1.f;
-        if (normalise) {
-            float ss = 0.f;
-            for (int d = lane; d < hd; d += KA_WAVE) {
-                const float v = ka_to_float(p[d]);
-                ss = fmaf(v, v, ss);
-            }
-            rinv = 1.0f / sqrtf(ka_wave_sum(ss) / (float)hd + eps);
-        }
-        const bool key = h >= H;
-        T* kdst = key && slot >= 0 ? k_cache + (((size_t)page * Hkv + (h - H)) * page_size + off) * hd : nullptr;
-        for (int d = lane; d < hd; d += KA_WAVE) {
-            const T y = ka_from_float<T>(ka_to_float(p[d]) * rinv);
-            if (normalise) p[d] = y;
-            if (kdst) kdst[d] = y;
-        }
+    if (h >= H + Hkv) {
+        if (slot < 0) return;
+        const int g = h - H - Hkv;
+        const T* vrow = row + (size_t)(H + Hkv) * hd + (size_t)g * hdv;
+        T* dst = v_cache + (((size_t)page * Hkv + g) * hdv) * page_size + off;
+        for (int d = lane; d < hdv; d += KA_WAVE) dst[(size_t)d * page_size] = vrow[d];
+        return;
     }
-    if (slot < 0) return;
-    const T* vrow = row + (size_t)(H + Hkv) * hd;
-    for (int idx = threadIdx.x; idx < Hkv * hdv; idx += blockDim.x) {
-        const int h = idx / hdv, d = idx % hdv;
-        v_cache[(((size_t)page * Hkv + h) * hdv + d) * page_size + off] = vrow[idx];
+    T* p = row + (size_t)h * hd;
+    const bool key = h >= H;
+    if (!normalise && !(key && slot >= 0)) return;
+    T* kdst = key && slot >= 0 ? k_cache + (((size_t)page * Hkv + (h - H)) * page_size + off) * hd : nullptr;
+    if (hd <= KA_WAVE) {
+        // the whole head in one load a lane
+        const float v = lane < hd ? ka_to_float(p[lane]) : 0.f;
+        const float rinv = normalise ? 1.0f / sqrtf(ka_wave_sum(v * v) / (float)hd + eps) : 1.f;
+        if (lane < hd) {
+            const T y = ka_from_float<T>(v * rinv);
+            if (normalise) p[lane] = y;
+            if (kdst) kdst[lane] = y;
+        }
+        return;
+    }
+    float rinv = 1.f;
+    if (normalise) {
+        float ss = 0.f;
+        for (int d = lane; d < hd; d += KA_WAVE) {
+            const float v = ka_to_float(p[d]);
+            ss = fmaf(v, v, ss);
+        }
+        rinv = 1.0f / sqrtf(ka_wave_sum(ss) / (float)hd + eps);
+    }
+    for (int d = lane; d < hd; d += KA_WAVE) {
+        const T y = ka_from_float<T>(ka_to_float(p[d]) * rinv);
+        if (normalise) p[d] = y;
+        if (kdst) kdst[d] = y;
     }
 }
 
@@ -514,7 +620,8 @@ KA_API int ka_unit_norm_cache(void* qkv, int dtype, long row_stride, const int* 
     KA_CHECK(page_size > 0 && eps >= 0.f, "ka_unit_norm_cache: page size %d, eps %g", page_size, eps);
     KA_CHECK(slots == nullptr || (k_cache && v_cache), "ka_unit_norm_cache: cache tensors missing");
     if (n == 0) return 0;
-    dim3 grid(n), block(256);
+    KA_CHECK((H + 2 * Hkv + 3) / 4 <= 65535, "ka_unit_norm_cache: too many heads");
+    dim3 grid(n, (H + 2 * Hkv + 3) / 4), block(256);
     if (dtype == KA_F32)
         hipLaunchKernelGGL(unit_norm_cache_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, slots,
                            (float*)k_cache, (float*)v_cache, H, Hkv, hd, hdv, page_size, eps, normalise);

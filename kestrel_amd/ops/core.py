@@ -35,7 +35,7 @@ _SIGNATURES = {
     "ka_add_table_rows": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_cast_columns": [_c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],
     "ka_add_scaled": [_c_void_p, _c_void_p, _c_float, _c_long, _c_void_p],
-    "ka_layernorm_pair": [_c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float,
+    "ka_layernorm_pair": [_c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float,
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "ka_unit_norm_cache": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                            _c_int, _c_int, _c_float, _c_int, _c_void_p],
@@ -254,10 +254,11 @@ def add_scaled(x: torch.Tensor, delta: torch.Tensor, scale: float) -> None:
 
 
 def layernorm_pair(x: torch.Tensor, first, second, out1: Optional[torch.Tensor], out2: Optional[torch.Tensor],
-                   delta: Optional[torch.Tensor] = None, scale: float = 1.0, apply: bool = False) -> None:
+                   delta: Optional[torch.Tensor] = None, scale: float = 1.0, apply: bool = False, clear: bool = True) -> None:
     """Two LayerNorms of the same fp32 rows in one pass: ``out1 = LN(x; first)`` and, if ``second`` is given,
     ``out2 = LN(x; second)``, each of ``first`` / ``second`` being ``(gamma, beta or None, eps)`` with one ``eps``.
-    ``delta`` (fp32, the shape of ``x``): cleared, after ``x += scale * delta`` if ``apply``. ``first`` ``None``: only that."""
+    ``delta`` (fp32, the shape of ``x``): ``x += scale * delta`` first if ``apply``, and ``delta`` is zeroed after that if
+    ``clear`` (for branches that add into it). ``first`` ``None``: only that."""
     _dev(x, out1, out2, delta)
     n, dim = x.shape
     _need(x.dtype == torch.float32 and x.is_contiguous(), "layernorm_pair: x must be contiguous fp32")
@@ -277,7 +278,11 @@ def layernorm_pair(x: torch.Tensor, first, second, out1: Optional[torch.Tensor],
             _need(t is None or (t.dtype == torch.float32 and t.numel() == dim and t.is_cuda), "layernorm_pair: gains and shifts fp32 [dim]")
     else:
         _need(second is None and delta is not None, "layernorm_pair: nothing to do")
-    _check(lib().ka_layernorm_pair(x.data_ptr(), _ptr(delta), float(scale), int(bool(apply)), _ptr(g1), _ptr(b1), _ptr(g2), _ptr(b2),
+    if delta is None:
+        apply = clear = False
+    if first is None and not (apply or clear):
+        return
+    _check(lib().ka_layernorm_pair(x.data_ptr(), _ptr(delta), float(scale), int(bool(apply)), int(bool(clear)), _ptr(g1), _ptr(b1), _ptr(g2), _ptr(b2),
                                    float(eps), _ptr(out1) if first is not None else None,
                                    _ptr(out2) if second is not None else None,
                                    code_of(out1.dtype) if first is not None else KA_F32, n, dim, stream_ptr()))

@@ -303,8 +303,9 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     return True
 
 
-def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out, then_norm=None) -> bool:
-    """``out += a1 @ w1.T + b1 + a2 @ w2.T + b2`` in one launch (few rows, fp32 ``out``).
+def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out, then_norm=None, accumulate: bool = True) -> bool:
+    """``out += a1 @ w1.T + b1 + a2 @ w2.T + b2`` in one launch (few rows, fp32 ``out``); with ``accumulate`` off
+    the sum replaces ``out``.
     ``then_norm = (gamma, beta or None, eps, normed)``: also ``normed = LayerNorm(out)``, in the kernel
     that finishes the rows where there is one (more than 8 rows), else in a launch behind it. False:
     not covered, nothing was run (with ``then_norm``: try without)."""
@@ -328,14 +329,14 @@ def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out, then_norm=None) -> bool:
             return False
         _check(lib().ka_linear_skinny_pair_norm(
             a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w1.data_ptr(), w1.stride(0), _ptr(b1),
-            w2.data_ptr(), w2.stride(0), _ptr(b2), out.data_ptr(), out.stride(0), n, 1, m, chip_sizes(a1.device).skinny_target_waves,
+            w2.data_ptr(), w2.stride(0), _ptr(b2), out.data_ptr(), out.stride(0), n, int(bool(accumulate)), m, chip_sizes(a1.device).skinny_target_waves,
             *_wide_args(a1.device, m), gamma.data_ptr(), _ptr(beta), float(eps), normed.data_ptr(), _OUT_CODE[normed.dtype],
             normed.stride(0), stream_ptr()))
         return True
     _check(lib().ka_linear_skinny_fused(
         a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w2.data_ptr(), w2.stride(0), _ptr(b2),
         None, None, None, 0.0,
-        w1.data_ptr(), w1.stride(0), _ptr(b1), out.data_ptr(), KA_F32, out.stride(0), n, 0, 1,
+        w1.data_ptr(), w1.stride(0), _ptr(b1), out.data_ptr(), KA_F32, out.stride(0), n, 0, int(bool(accumulate)),
         None, 0, None, None, 0, 0, 0, 0, m, chip_sizes(a1.device).skinny_target_waves, *_wide_args(a1.device, m), stream_ptr()))
     return True
 

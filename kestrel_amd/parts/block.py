@@ -121,28 +121,32 @@ def settle(x, batch) -> None:
         core.add_scaled(x, pending[0], pending[1])
 
 
-def _two_branches_few_rows(block: "Block", h1, h2, batch, cache, delta) -> bool:
-    """Both branches for a few bf16 rows: the two first linears, the mixer's core, and both last linears adding into
-    ``delta`` in one launch. Needs a mixer and a feed-forward that offer their stages; ``False`` otherwise."""
+def _two_branches_by_stages(block: "Block", h1, h2, batch, cache, delta) -> bool:
+    """Both branches through the stages that mixer and feed-forward offer, so that the first of the last linears
+    writes ``delta`` and nobody has to clear it: for a few bf16 rows the two last linears are one launch.
+    ``False``: a part offers no stages (its ``forward`` then adds into a cleared ``delta``)."""
     from ..ops import fast
     from ..ops.linear import linear
 
     n = h1.shape[0]
     ff = block.feed_forward
-    if ff is None or block.dtype != torch.bfloat16 or n > fast.SKINNY_MAX_ROWS:
-        return False
-    m_in, f_in = block.mixer.input_projection(), ff.input_projection()
-    m_out, f_out = block.mixer.output_projection(), ff.output_projection()
-    if m_in is None or f_in is None or m_out is None or f_out is None:
+    m_in, m_out = block.mixer.input_projection(), block.mixer.output_projection()
+    f_in, f_out = (ff.input_projection(), ff.output_projection()) if ff is not None else (None, None)
+    if m_in is None or m_out is None or (ff is not None and (f_in is None or f_out is None)):
         return False
     ws = batch.workspace
     projected = ws.get("block.mixer_in", (n, m_in[2]), block.dtype)
-    hidden = ws.get("block.ff_hidden", (n, f_in[2]), block.dtype)
     linear(h1, m_in[0], m_in[1], projected)
-    linear(h2, f_in[0], f_in[1], hidden, act=f_in[3])
+    hidden = None
+    if ff is not None:
+        hidden = ws.get("block.ff_hidden", (n, f_in[2]), block.dtype)
+        linear(h2, f_in[0], f_in[1], hidden, act=f_in[3])
     mixed = block.mixer.attend(projected, batch, cache)
-    if not fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], delta):
-        linear(mixed, m_out[0], m_out[1], delta, accumulate=True)
+    if ff is not None and block.dtype == torch.bfloat16 and n <= fast.SKINNY_MAX_ROWS and \
+            fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], delta, accumulate=False):
+        return True
+    linear(mixed, m_out[0], m_out[1], delta)
+    if ff is not None:
         linear(hidden, f_out[0], f_out[1], delta, accumulate=True)
     return True
 
@@ -152,8 +156,8 @@ def _parallel_two_norms(block: "Block", x, batch, cache) -> None:
     same ``x``; without a feed-forward, ``x + residual_scale * mixer(norm(x))``.
 
     Both norms come from one pass over ``x`` where they are LayerNorms of one eps; that pass also adds what the
-    block before has left to be added (``DEFER_RESIDUAL``) and clears the buffer the branches add into. The
-    branches' sum enters the stream with the weight in fp32, like the stream."""
+    block before has left to be added (``DEFER_RESIDUAL``). The branches' sum is kept in a buffer of its own and
+    enters the stream with the weight in fp32, like the stream."""
     from ..ops import core
 
     ws = batch.workspace
@@ -163,24 +167,30 @@ def _parallel_two_norms(block: "Block", x, batch, cache) -> None:
     ln1 = block.norm.layernorm_operands()
     ln2 = block.norm2.layernorm_operands() if ff is not None else None
     h2 = ws.get("block.h2", tuple(x.shape), block.dtype) if ff is not None else None
-    pending = batch.host.get(_PENDING)
+    host = batch.host
+    pending = host.get(_PENDING)
     if pending is not None and pending[0].data_ptr() != delta.data_ptr():
         settle(x, batch)              # (left in another buffer than this block's)
         pending = None
+    # parts that offer their stages write the buffer; parts that only add need it cleared
+    staged = block.mixer.input_projection() is not None and block.mixer.output_projection() is not None and \
+        (ff is None or (ff.input_projection() is not None and ff.output_projection() is not None))
+    sum_args = dict(delta=delta if (pending is not None or not staged) else None, scale=pending[1] if pending else 1.0,
+                    apply=pending is not None, clear=not staged)
     if ln1 is not None and (ff is None or (ln2 is not None and float(ln2[2]) == float(ln1[2]))):
-        core.layernorm_pair(x, ln1, ln2, h1, h2, delta=delta, scale=pending[1] if pending else 1.0, apply=pending is not None)
+        core.layernorm_pair(x, ln1, ln2, h1, h2, **sum_args)
     else:
-        core.layernorm_pair(x, None, None, None, None, delta=delta, scale=pending[1] if pending else 1.0, apply=pending is not None)
+        core.layernorm_pair(x, None, None, None, None, **sum_args)
         block.norm.forward(x, h1)
         if ff is not None:
             block.norm2.forward(x, h2)
-    batch.host.pop(_PENDING, None)
-    if not _two_branches_few_rows(block, h1, h2, batch, cache, delta):
+    host.pop(_PENDING, None)
+    if not (staged and _two_branches_by_stages(block, h1, h2, batch, cache, delta)):
         block.mixer.forward(h1, batch, cache, delta)
         if ff is not None:
             ff.forward(h2, batch, delta)
     if DEFER_RESIDUAL:
-        batch.host[_PENDING] = (delta, float(block.spec.residual_scale))
+        host[_PENDING] = (delta, float(block.spec.residual_scale))
     else:
         core.add_scaled(x, delta, block.spec.residual_scale)
 
