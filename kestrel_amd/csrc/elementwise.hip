@@ -564,12 +564,13 @@ KA_API int ka_layernorm_pair(float* x, float* delta, float scale, int apply, int
 template <typename T>
 __global__ void __launch_bounds__(256)
 unit_norm_cache_kernel(T* __restrict__ qkv, long row_stride, const int* __restrict__ slots, T* __restrict__ k_cache,
-                       T* __restrict__ v_cache, int H, int Hkv, int hd, int hdv, int page_size, float eps, int normalise) {
-    // a wave per head of a token: the query heads, then the key heads, then the value heads
+                       T* __restrict__ v_cache, int H, int Hkv, int hd, int hdv, int page_size, float eps, int normalise,
+                       int with_values) {
+    // a wave per head of a token: the query heads, then the key heads, then (with_values) the value heads
     const int t = blockIdx.x;
     const int lane = threadIdx.x % KA_WAVE;
     const int h = blockIdx.y * (blockDim.x / KA_WAVE) + threadIdx.x / KA_WAVE;
-    if (h >= H + 2 * Hkv) return;
+    if (h >= H + (with_values ? 2 : 1) * Hkv) return;
     T* row = qkv + (size_t)t * row_stride;
     const long slot = slots ? slots[t] : -1;
     const long page = slot >= 0 ? slot / page_size : 0, off = slot >= 0 ? slot % page_size : 0;
@@ -612,22 +613,128 @@ unit_norm_cache_kernel(T* __restrict__ qkv, long row_stride, const int* __restri
     }
 }
 
+// The same for bf16 heads of a multiple of 8 channels on 16-byte aligned rows: a lane holds a 16-byte chunk of a head,
+// LPH lanes (the next power of two of hd / 8) a head, 64 / LPH heads a wave; the sum of squares meets inside those lanes.
+// Query and key heads only (the values go run by run, or through the kernel above).
+template <int LPH>
+__global__ void __launch_bounds__(256)
+unit_norm_cache_chunks_kernel(bf16_t* __restrict__ qkv, long row_stride, const int* __restrict__ slots,
+                              bf16_t* __restrict__ k_cache, int H, int Hkv, int hd, int page_size, float eps, int normalise) {
+    typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+    const int t = blockIdx.x;
+    const int lane = threadIdx.x % KA_WAVE;
+    const int h = (blockIdx.y * (blockDim.x / KA_WAVE) + threadIdx.x / KA_WAVE) * (KA_WAVE / LPH) + lane / LPH;
+    const int c = (lane % LPH) * 8;
+    const bool live = h < H + Hkv && c < hd;
+    bf16_t* p = qkv + (size_t)t * row_stride + (size_t)(live ? h : 0) * hd + (live ? c : 0);
+    bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
+    float f[8], ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        f[e] = live ? (float)v[e] : 0.f;
+        ss = fmaf(f[e], f[e], ss);
+    }
+    ss = ka_lanes_reduce<1, LPH>(ss, KaSum{});
+    if (!live) return;
+    const float rinv = normalise ? 1.0f / sqrtf(ss / (float)hd + eps) : 1.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (bf16_t)(f[e] * rinv);
+    if (normalise) *reinterpret_cast<bf16x8*>(p) = v;
+    const long slot = slots ? slots[t] : -1;
+    if (h >= H && slot >= 0)
+        *reinterpret_cast<bf16x8*>(k_cache + (((size_t)(slot / page_size) * Hkv + (h - H)) * page_size + slot % page_size) * hd + c) = v;
+}
+
+// The values of runs of tokens into the cache. A run is `count` neighbouring tokens of the packed batch (at most a
+// page's worth); one that fills a page of its row in order (count == page_size, the first at a page's start, the
+// slots consecutive) is turned through LDS and leaves as the page's contiguous [hdv][page_size] block; any other
+// run goes token by token. One workgroup per (run, kv head).
+constexpr int UN_MAX_TILE = 16 * 520;            // page 16, value heads of up to 512 channels (+ padding)
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+value_cache_runs_kernel(const T* __restrict__ qkv, long row_stride, long v_offset, const int* __restrict__ slots,
+                        const int* __restrict__ run_first, const int* __restrict__ run_count, T* __restrict__ v_cache,
+                        int Hkv, int hdv, int page_size) {
+    __shared__ T tile[UN_MAX_TILE];
+    const int count = run_count[blockIdx.x];
+    if (count <= 0) return;
+    const int first = run_first[blockIdx.x], g = blockIdx.y;
+    const int s0 = slots[first];
+    const int pitch = hdv + 2;
+    const bool whole = count == page_size && page_size == 16 && s0 >= 0 && s0 % page_size == 0 &&
+                       slots[first + count - 1] == s0 + count - 1 && page_size * pitch <= UN_MAX_TILE;
+    if (whole) {
+        for (int idx = threadIdx.x; idx < page_size * hdv; idx += blockDim.x) {
+            const int i = idx / hdv, d = idx % hdv;
+            tile[i * pitch + d] = qkv[(size_t)(first + i) * row_stride + v_offset + (size_t)g * hdv + d];
+        }
+        __syncthreads();
+        T* dst = v_cache + (((size_t)(s0 / page_size) * Hkv + g) * hdv) * page_size;
+        for (int idx = threadIdx.x; idx < page_size * hdv; idx += blockDim.x) {
+            const int d = idx / page_size, i = idx % page_size;
+            dst[idx] = tile[i * pitch + d];
+        }
+        return;
+    }
+    for (int idx = threadIdx.x; idx < count * hdv; idx += blockDim.x) {
+        const int i = idx / hdv, d = idx % hdv;
+        const long slot = slots[first + i];
+        if (slot < 0) continue;
+        v_cache[(((size_t)(slot / page_size) * Hkv + g) * hdv + d) * page_size + slot % page_size] =
+            qkv[(size_t)(first + i) * row_stride + v_offset + (size_t)g * hdv + d];
+    }
+}
+
+// run_first / run_count (optional, n_runs of them): the tokens cut into runs, every token in exactly one and none
+// longer than a page; the values then go into the cache run by run (whole pages as contiguous blocks).
 KA_API int ka_unit_norm_cache(void* qkv, int dtype, long row_stride, const int* slots, void* k_cache, void* v_cache,
                               int n, int H, int Hkv, int hd, int hdv, int page_size, float eps, int normalise,
-                              hipStream_t stream) {
+                              const int* run_first, const int* run_count, int n_runs, hipStream_t stream) {
     KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0 && hdv > 0, "ka_unit_norm_cache: bad sizes");
     KA_CHECK(row_stride >= (long)(H + Hkv) * hd + (long)Hkv * hdv, "ka_unit_norm_cache: row stride %ld too small", row_stride);
     KA_CHECK(page_size > 0 && eps >= 0.f, "ka_unit_norm_cache: page size %d, eps %g", page_size, eps);
     KA_CHECK(slots == nullptr || (k_cache && v_cache), "ka_unit_norm_cache: cache tensors missing");
     if (n == 0) return 0;
     KA_CHECK((H + 2 * Hkv + 3) / 4 <= 65535, "ka_unit_norm_cache: too many heads");
-    dim3 grid(n, (H + 2 * Hkv + 3) / 4), block(256);
+    const bool by_runs = slots && run_first && run_count && n_runs > 0 && Hkv <= 65535;
+    // (with the values written run by run, the first launch ends with the key heads: the kernel passes over heads
+    // behind H + 2 Hkv, so it is told of no value heads at all by way of its grid)
+    dim3 grid(n, ((by_runs ? H + Hkv : H + 2 * Hkv) + 3) / 4), block(256);
+    if (by_runs) {
+        dim3 rgrid(n_runs, Hkv);
+        const long v_offset = (long)(H + Hkv) * hd;
+        if (dtype == KA_F32)
+            hipLaunchKernelGGL(value_cache_runs_kernel<float>, rgrid, block, 0, stream, (const float*)qkv, row_stride, v_offset,
+                               slots, run_first, run_count, (float*)v_cache, Hkv, hdv, page_size);
+        else if (dtype == KA_BF16)
+            hipLaunchKernelGGL(value_cache_runs_kernel<bf16_t>, rgrid, block, 0, stream, (const bf16_t*)qkv, row_stride, v_offset,
+                               slots, run_first, run_count, (bf16_t*)v_cache, Hkv, hdv, page_size);
+    }
+    // bf16 heads in 16-byte chunks where rows and heads are aligned for it (the values then go run by run, or, without
+    // runs, through a launch of the plain kernel that starts behind the key heads: here the plain kernel does it all)
+    const int chunks = hd / 8;
+    if (dtype == KA_BF16 && by_runs && hd % 8 == 0 && chunks <= 64 && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0 &&
+        (uintptr_t)k_cache % 16 == 0) {
+        int lph = 1;
+        while (lph < chunks) lph *= 2;
+        const int heads_per_block = 4 * (KA_WAVE / lph);
+        dim3 cgrid(n, (H + Hkv + heads_per_block - 1) / heads_per_block);
+#define KA_UN_CHUNKS(LPH)                                                                                                  \
+    if (lph == LPH)                                                                                                        \
+        hipLaunchKernelGGL(unit_norm_cache_chunks_kernel<LPH>, cgrid, block, 0, stream, (bf16_t*)qkv, row_stride, slots,   \
+                           (bf16_t*)k_cache, H, Hkv, hd, page_size, eps, normalise)
+        KA_UN_CHUNKS(1); KA_UN_CHUNKS(2); KA_UN_CHUNKS(4); KA_UN_CHUNKS(8); KA_UN_CHUNKS(16); KA_UN_CHUNKS(32); KA_UN_CHUNKS(64);
+#undef KA_UN_CHUNKS
+        KA_LAUNCH_CHECK();
+        return 0;
+    }
     if (dtype == KA_F32)
         hipLaunchKernelGGL(unit_norm_cache_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, slots,
-                           (float*)k_cache, (float*)v_cache, H, Hkv, hd, hdv, page_size, eps, normalise);
+                           (float*)k_cache, (float*)v_cache, H, Hkv, hd, hdv, page_size, eps, normalise, by_runs ? 0 : 1);
     else if (dtype == KA_BF16)
         hipLaunchKernelGGL(unit_norm_cache_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, row_stride, slots,
-                           (bf16_t*)k_cache, (bf16_t*)v_cache, H, Hkv, hd, hdv, page_size, eps, normalise);
+                           (bf16_t*)k_cache, (bf16_t*)v_cache, H, Hkv, hd, hdv, page_size, eps, normalise, by_runs ? 0 : 1);
     else
         KA_CHECK(false, "ka_unit_norm_cache: unsupported dtype %d", dtype);
     KA_LAUNCH_CHECK();

@@ -38,7 +38,7 @@ _SIGNATURES = {
     "ka_layernorm_pair": [_c_void_p, _c_void_p, _c_float, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float,
                           _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "ka_unit_norm_cache": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
-                           _c_int, _c_int, _c_float, _c_int, _c_void_p],
+                           _c_int, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
     "ka_argmax": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
     "ka_suppress_tokens": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_allow_tokens": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
@@ -290,11 +290,13 @@ def layernorm_pair(x: torch.Tensor, first, second, out1: Optional[torch.Tensor],
 
 def unit_norm_cache(qkv: torch.Tensor, slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
                     v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int,
-                    page_size: int, eps: Optional[float]) -> None:
+                    page_size: int, eps: Optional[float], runs=None) -> None:
     """Divide every query and key head of ``qkv`` ``[n, H hd | Hkv hd | Hkv hdv]`` by its root mean square
     (``x / sqrt(mean(x^2) + eps)``, in place; ``eps`` ``None``: left as they are) and write keys and values into the
     paged cache (keys ``[pages, Hkv, page_size, hd]``, values ``[pages, Hkv, hdv, page_size]``; ``slots`` ``None``
-    writes nothing)."""
+    writes nothing). ``runs``: (int32 first token, int32 count) of the runs the tokens are cut into, every token in
+    exactly one and none longer than a page (``StepBatch.page_runs``): values of a run that fills a page leave as
+    the page's contiguous block."""
     _dev(qkv, slots, k_cache, v_cache)
     n = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim,
@@ -303,9 +305,15 @@ def unit_norm_cache(qkv: torch.Tensor, slots: Optional[torch.Tensor], k_cache: O
         _need(slots.dtype == torch.int32 and slots.numel() == n and slots.is_contiguous(), "unit_norm_cache: slots int32 [n]")
         _need(k_cache is not None and v_cache is not None, "unit_norm_cache: cache tensors missing")
         _check_caches("unit_norm_cache", k_cache, v_cache, qkv.dtype, n_kv_heads, page_size, head_dim, value_dim)
+    first, count = runs if (runs is not None and slots is not None) else (None, None)
+    if first is not None:
+        _dev(first, count)
+        _need(first.dtype == torch.int32 and count.dtype == torch.int32 and first.numel() == count.numel()
+              and first.is_contiguous() and count.is_contiguous(), "unit_norm_cache: runs are two int32 lists of one length")
     _check(lib().ka_unit_norm_cache(qkv.data_ptr(), code_of(qkv.dtype), qkv.stride(0) if n > 1 else qkv.shape[1], _ptr(slots),
                                     _ptr(k_cache), _ptr(v_cache), n, n_heads, n_kv_heads, head_dim, value_dim, page_size,
-                                    float(eps or 0.0), int(eps is not None), stream_ptr()))
+                                    float(eps or 0.0), int(eps is not None), _ptr(first), _ptr(count),
+                                    int(first.numel()) if first is not None else 0, stream_ptr()))
 
 
 ROTARY_PAIRINGS = {"halves": 0, "interleaved": 1}

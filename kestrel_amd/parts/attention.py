@@ -194,8 +194,10 @@ class PagedAttention(Mixer):
         """Queries and keys to unit norm, the cache write, then attention with the terms the specification names."""
         spec = self.spec
         slots = group.slots if cache.writes else None
+        # (a decode step's tokens are each a run of their own: nothing to gain from the lists there)
         core.unit_norm_cache(qkv, slots, cache.k, cache.v, spec.n_heads, spec.n_kv_heads, spec.head_dim, self.value_dim,
-                             group.page_size, self.unit_norm_eps)
+                             group.page_size, self.unit_norm_eps,
+                             runs=None if batch.decode_only else getattr(batch, "page_runs", None))
         if qkv.dtype == torch.bfloat16:
             from ..ops import fast
             if fast.attention_biased_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi,

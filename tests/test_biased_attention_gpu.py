@@ -216,6 +216,21 @@ def test_unit_norm_and_cache_write(dtype):
         assert torch.allclose(k_cache[page, :, off].double().cpu(), want_qk[t, heads:], atol=tol, rtol=tol)
         assert torch.equal(v_cache[page, :, :, off].double().cpu(), x[t, (heads + kv_heads) * d:].reshape(kv_heads, dv))
     assert float(k_cache.abs().sum(dim=(1, 3)).ne(0).sum()) == n - 1
+    # the same tokens cut into runs: 16 tokens that fill a page in order leave as the page's block, the others one by one
+    ordered = torch.cat([torch.arange(32, 48), torch.tensor([5, 70, 71, 3]), torch.arange(80, 96), torch.tensor([20])]).to(torch.int32)
+    first = torch.tensor([0, 16, 20, 36, 37], dtype=torch.int32)          # (the last run is empty: a list of fixed length)
+    count = torch.tensor([16, 4, 16, 1, 0], dtype=torch.int32)
+    k2, v2 = torch.zeros_like(k_cache), torch.zeros_like(v_cache)
+    dev2 = qkv.to(DEV).clone()
+    core.unit_norm_cache(dev2, ordered.to(DEV), k2, v2, heads, kv_heads, d, dv, PAGE, eps, runs=(first.to(DEV), count.to(DEV)))
+    k3, v3 = torch.zeros_like(k_cache), torch.zeros_like(v_cache)
+    dev3 = qkv.to(DEV).clone()
+    core.unit_norm_cache(dev3, ordered.to(DEV), k3, v3, heads, kv_heads, d, dv, PAGE, eps)
+    torch.cuda.synchronize()
+    # (bf16 with runs takes the form that moves 16 bytes a lane: its sums run in another order, a last bit may differ)
+    assert torch.equal(v2, v3) and float(v2.abs().sum()) > 0
+    assert torch.allclose(k2.float(), k3.float(), atol=tol, rtol=tol) and torch.allclose(dev2.float(), dev3.float(), atol=tol, rtol=tol)
+    assert torch.allclose(dev2.double().cpu()[:, :(heads + kv_heads) * d].reshape(n, -1, d), want_qk, atol=tol, rtol=tol)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
