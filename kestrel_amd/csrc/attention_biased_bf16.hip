@@ -219,7 +219,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     }
     l = ab_sum_halves(l);                       // the column's whole sum, in both of its lanes
 
-    // merge the waves in a tree: in round r the waves with bit r set hand over to the wave 2^r below
+    // merge the waves in a tree: at step s the waves with bit s set hand over to the wave 2^s below
     for (int step = 1; step < n_waves; step <<= 1) {
         const bool gives = (wave & (2 * step - 1)) == step, takes = (wave & (2 * step - 1)) == 0 && wave + step < n_waves;
         float* slot = mrg + (size_t)(wave / (2 * step)) * REC * KA_WAVE;
