@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DTYPES = [torch.float32, torch.bfloat16]
 DTYPE_IDS = ["fp32", "bf16"]
-NAMES = ["P", "Q", "R", "S"]
+NAMES = ["P", "Q", "R", "S", "T"]
 
 
 def _runner(folder, dtype, n_pages=64, max_requests=4, graphs=False):

@@ -39,9 +39,13 @@ CONFIGS: Dict[str, dict] = {
     "R": _config(257, 128, 400, 1e-5, 0.8, [_layer(6, 3, 32, 96, 0.2, None, 136), _layer(6, 3, 32, 96, 0.2, 1000, 136)]),
     # the largest head sizes of the matrix-core kernel, a loop that ends with the stack, two passes
     "S": _config(190, 256, 320, 1e-5, 0.6, [_layer(4, 1, 128, 128, 0.09, 50, 264), _layer(2, 2, 96, 112, 0.1, 33, 264)], (1, 2, 2)),
+    # sizes that fit none of the fast kernels' alignments: an odd width, head sizes that are no multiple of 8 or of 4, five
+    # heads, an odd feed-forward and vocabulary; three passes over the first two layers, the stack ending outside the loop
+    "T": _config(77, 100, 260, 1e-5, 0.9, [_layer(5, 5, 24, 10, 0.3, 19, 50), _layer(6, 2, 20, 36, 0.25, 64, None),
+                                           _layer(1, 1, 40, 44, 0.2, 33, 90)], (0, 2, 3)),
 }
 RECIPE = InitRecipe(std=0.08, gain_std=0.1, shift_std=0.05)
-SEEDS = {"P": 11, "Q": 12, "R": 13, "S": 14}
+SEEDS = {"P": 11, "Q": 12, "R": 13, "S": 14, "T": 15}
 
 
 @functools.lru_cache(maxsize=None)
