@@ -113,7 +113,7 @@ def compare_models(size: dict, positions: int):
     else:
         mixer["mask"] = {"size": positions}
     vimesun = {"architecture": "Vimesun", "vocab": COMPARE_VOCAB, "width": size["width"], "max_positions": positions,
-               "norm": {"eps": 1e-5}, "residual_mult": 0.7, "loop": dict(zip(("start", "stop", "times"), size["loop"])),
+               "norm": {"eps": 1e-5}, "residual_mult": 0.5, "loop": dict(zip(("start", "stop", "times"), size["loop"])),
                "layers": [{"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": size["ff"]}}
                           for _ in range(size["layers"])]}
     moondream = {"text": {"dim": size["width"], "ff_dim": size["ff"], "n_layers": runs, "vocab_size": COMPARE_VOCAB,

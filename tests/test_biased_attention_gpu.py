@@ -128,7 +128,7 @@ def test_decode_steps(kernel, dtype, heads, kv_heads, d, dv):
     """One token per row (the kernel then puts the heads that share a kv head side by side), rows of very different
     lengths, also a row of one token."""
     lengths = [1, 2, 16, 17, 33, 250, 129, 700]
-    for window in (None, 136, 16):
+    for window in (None, 120, 16):
         case = Case(dtype, heads, kv_heads, d, dv, lengths=lengths, starts=[n - 1 for n in lengths], window=window, seed=d + dv)
         assert case.batch().decode_only
         _close(_run(case, 0.21, kernel), case.expected(0.21), dtype, f"window {window}")
@@ -152,8 +152,8 @@ def _point_at(distance_of):
 def test_one_key_that_stands_out(kernel, dtype, mode):
     """A key far back, the last one inside the window, the first one outside it, keys at page borders, the first
     token of the sequence: the query points at it with a score that dwarfs the others'."""
-    window, scale, d = 136, 1.5, 32          # a matching key scores 1.5 * 32 = 48, the others around 1.5 * sqrt(32)
-    lengths = [400, 277, 150, 137, 136]
+    window, scale, d = 120, 1.5, 32          # a matching key scores 1.5 * 32 = 48, the others around 1.5 * sqrt(32)
+    lengths = [400, 277, 150, 121, 120]
     starts = [0] * len(lengths) if mode == "prompt" else [n - 1 for n in lengths]
     for what, distance in (("far", lambda p: p - 3 if window is None else min(p, window - 6)),
                            ("last inside", lambda p: window - 1), ("first outside", lambda p: window),
@@ -245,9 +245,9 @@ def test_two_norms_in_one_pass_and_the_weighted_sum(dtype):
     xd, dd = x.to(DEV), delta.to(DEV)
     out1 = torch.empty(n, dim, dtype=dtype, device=DEV)
     out2 = torch.empty(n, dim, dtype=dtype, device=DEV)
-    core.layernorm_pair(xd, (g1.to(DEV), b1.to(DEV), eps), (g2.to(DEV), b2.to(DEV), eps), out1, out2, delta=dd, scale=0.7, apply=True)
+    core.layernorm_pair(xd, (g1.to(DEV), b1.to(DEV), eps), (g2.to(DEV), b2.to(DEV), eps), out1, out2, delta=dd, scale=0.45, apply=True)
     torch.cuda.synchronize()
-    summed = x.double() + 0.7 * delta.double()
+    summed = x.double() + 0.45 * delta.double()
     assert torch.allclose(xd.double().cpu(), summed, atol=1e-6) and float(dd.abs().max()) == 0.0
     tol = 2e-5 if dtype == torch.float32 else 3e-2
     assert torch.allclose(out1.double().cpu(), plain.layer_norm(summed, g1.double(), b1.double(), eps), atol=tol, rtol=tol)
@@ -258,7 +258,7 @@ def test_two_norms_in_one_pass_and_the_weighted_sum(dtype):
     assert torch.allclose(out1.double().cpu(), plain.layer_norm(summed, g1.double(), torch.zeros(dim, dtype=torch.float64), eps), atol=tol, rtol=tol)
     assert float(dd.abs().max()) == 0.0 and torch.allclose(xd.double().cpu(), summed, atol=1e-6)
     dd.copy_(delta)
-    core.add_scaled(xd, dd, -0.7)
+    core.add_scaled(xd, dd, -0.45)
     assert torch.allclose(xd.double().cpu(), x.double(), atol=1e-5)
 
 
@@ -293,7 +293,7 @@ def test_relu_squared_in_every_linear_kernel(rows, dtype):
     from kestrel_amd.ops.linear import activation_code, linear
 
     torch.manual_seed(rows)
-    k, n = 96, 136
+    k, n = 96, 152
     a = torch.randn(rows, k).to(dtype)
     w = (torch.randn(n, k) * 0.2).to(dtype)
     out = torch.empty(rows, n, dtype=dtype, device=DEV)

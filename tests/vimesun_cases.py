@@ -36,7 +36,7 @@ CONFIGS: Dict[str, dict] = {
     "Q": _config(211, 96, 300, 1e-6, 1.0, [_layer(2, 2, 48, 32, 0.3, 7, None), _layer(8, 1, 16, 20, 0.5, 200, 72),
                                             _layer(3, 1, 64, 64, 0.2, 1, 200)], (0, 3, 1)),
     # no loop at all, a layer without a window, a window longer than any sequence of the tests
-    "R": _config(257, 128, 400, 1e-5, 0.8, [_layer(6, 3, 32, 96, 0.2, None, 136), _layer(6, 3, 32, 96, 0.2, 1000, 136)]),
+    "R": _config(257, 128, 400, 1e-5, 0.8, [_layer(6, 3, 32, 96, 0.2, None, 152), _layer(6, 3, 32, 96, 0.2, 1000, 152)]),
     # the largest head sizes of the matrix-core kernel, a loop that ends with the stack, two passes
     "S": _config(190, 256, 320, 1e-5, 0.6, [_layer(4, 1, 128, 128, 0.09, 50, 264), _layer(2, 2, 96, 112, 0.1, 33, 264)], (1, 2, 2)),
     # sizes that fit none of the fast kernels' alignments: an odd width, head sizes that are no multiple of 8 or of 4, five
