@@ -27,6 +27,22 @@ from ..parts.base import LayerCache
 from ..parts.specs import CacheSpec, StateSpec
 
 
+def first_visible(spec, position: int) -> int:
+    """The lowest key position that a query at ``position`` reads under a cache specification: its own
+    ``first_visible`` if it has one (a window, chunks), else what its ``window`` says."""
+    own = getattr(spec, "first_visible", None)
+    if callable(own):
+        return int(own(position))
+    window = getattr(spec, "window", None)
+    return 0 if window is None else max(0, position + 1 - window)
+
+
+def reach(spec) -> Optional[int]:
+    """The most positions back (the query's own included) that any query reads, or ``None`` if there is no bound."""
+    spans = [s for s in (getattr(spec, "window", None), getattr(spec, "chunk", None)) if s is not None]
+    return min(spans) if spans else None
+
+
 class OutOfPages(RuntimeError):
     """A group's pool cannot back the positions asked for."""
 
@@ -177,7 +193,7 @@ class CacheManager:
         """Pages a request of ``length`` tokens holds at most in ``group`` when it is fed in
         portions of at most ``portion`` tokens."""
         full = -(-length // self.page_size)
-        window = self.groups[group].spec.window
+        window = reach(self.groups[group].spec)
         if window is None:
             return full
         # live keys span at most window - 1 + portion positions, which touch one page more
@@ -257,10 +273,9 @@ class CacheManager:
         state = self._slots[slot]
         freed = 0
         for g, grp in enumerate(self.groups):
-            window = grp.spec.window
-            if window is None:
+            if reach(grp.spec) is None:
                 continue
-            first_needed = max(0, length + 1 - window)        # lowest key the next query reads
+            first_needed = first_visible(grp.spec, length)    # lowest key the next query reads
             dead_below = min(first_needed // self.page_size, len(state.tables[g]))
             before = self._owed(state, g)
             dead = []
@@ -302,8 +317,7 @@ class CacheManager:
         return page * self.page_size + position % self.page_size
 
     def window_start(self, group: int, position: int) -> int:
-        window = self.groups[group].spec.window
-        return 0 if window is None else max(0, position + 1 - window)
+        return first_visible(self.groups[group].spec, position)
 
     # ------------------------------------------------------------------ invariants
     def check(self) -> None:

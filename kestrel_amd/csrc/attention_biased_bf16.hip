@@ -8,7 +8,8 @@
 // keys come normalised where the mixer normalises them.
 //
 // The score of query t (place p = positions[t]) of head h against the key at place j is
-//     scale * (q . k) - slopes[h] * (p - j)          (slopes optional)
+//     scale * (q . k) - slopes[h] * (p - j) + table[h, min(p - j, bias_len - 1)]     (slopes and table optional)
+// (the table: a learned bias per head and distance that is constant from some distance on, fp32 [H, bias_len]);
 // and the weights are exp(s_j) / (sum_j exp(s_j) [+ exp(sink)]): fp32 throughout; the weights enter
 // the value product as bf16, sums in fp32.
 //
@@ -58,7 +59,7 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo, const int* __restrict__ kv_hi,
                    const int* __restrict__ positions, const float* __restrict__ slopes, bf16_t* __restrict__ out,
                    long out_row_stride, float scale, int H, int Hkv, int hdv, int heads_per_block, int has_sink,
-                   float sink_score) {
+                   float sink_score, const float* __restrict__ bias_table, int bias_len) {
     constexpr int HD = NK * 16;
     constexpr int REC = 16 * NV + 2;            // floats a lane hands over at a merge: its outputs, m and l
     extern __shared__ float mrg[];              // [waves / 2][REC][64]
@@ -108,7 +109,9 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     }
     const float slope2 = slopes ? slopes[head] * AB_LOG2E : 0.f;     // in powers of two, like everything below
     const float scale2 = scale * AB_LOG2E;
-    const int place = slopes ? positions[tok] : 0;
+    const int place = (slopes || bias_table) ? positions[tok] : 0;
+    const float* bias_row = bias_table ? bias_table + (size_t)head * bias_len : nullptr;
+    const float bias_far2 = bias_row ? bias_row[bias_len - 1] * AB_LOG2E : 0.f;
     const float sink2 = sink_score * AB_LOG2E;
 
     float m = has_sink ? sink2 : -INFINITY;     // reference point of this lane's column (the same in both halves)
@@ -177,11 +180,16 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                         }
                     }
             }
+            // a tile that lies, for every column, at least as far back as the table's last entry: one bias for all its keys
+            const bool near_tile = bias_row != nullptr &&
+                __builtin_amdgcn_ballot_w64(place - (base + AB_TILE - 1) < bias_len - 1) != 0;
             float tile_max = -INFINITY;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int off = (i / 8) * 16 + i % 8;
                 float x = fmaf(s[i], scale2, fmaf(slope2, (float)off, bias0));
+                if (near_tile) x = fmaf(bias_row[min(max(place - (j0 + off), 0), bias_len - 1)], AB_LOG2E, x);
+                else x += bias_far2;
                 if (!whole) {
                     const int j = j0 + off;
                     if (j < lo || j >= hi) x = -INFINITY;
@@ -297,7 +305,8 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                                     int n_blocks, const int* cu_q, const int* token_row, const int* kv_lo,
                                     const int* kv_hi, const int* positions, const float* slopes, void* out,
                                     long out_row_stride, float scale, int n, int H, int Hkv, int hd, int hdv,
-                                    int page_size, int waves, int has_sink, float sink_score, hipStream_t stream) {
+                                    int page_size, int waves, int has_sink, float sink_score, const float* bias_table,
+                                    int bias_len, hipStream_t stream) {
     const char* who = "ka_attention_biased_bf16";
     KA_CHECK(n >= 0 && n_blocks >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes", who);
     KA_CHECK(page_size == AB_PAGE && ab_sizes_covered(hd, hdv), "%s: head sizes %d / %d or page size %d not covered", who, hd, hdv, page_size);
@@ -307,6 +316,7 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
              "%s: operands must be 16-byte aligned", who);
     KA_CHECK((uintptr_t)out % 8 == 0 && out_row_stride % 4 == 0, "%s: output rows must be 8-byte aligned", who);
     KA_CHECK(slopes == nullptr || positions != nullptr, "%s: slopes need the queries' positions", who);
+    KA_CHECK(bias_table == nullptr || (positions != nullptr && bias_len > 0), "%s: a distance table needs the queries' positions", who);
     KA_CHECK(n_blocks == 0 || (qblk_row && qblk_tok && cu_q), "%s: blocks of queries need their lists", who);
     if (n == 0) return 0;
     const int G = H / Hkv;
@@ -333,7 +343,7 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
         hipLaunchKernelGGL((attn_biased_kernel<NK, NV>), grid, dim3(KA_WAVE * waves), lds, stream, (const bf16_t*)q,       \
                            q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, \
                            qblk_tok, cu_q, token_row, kv_lo, kv_hi, positions, slopes, (bf16_t*)out, out_row_stride, scale, \
-                           H, Hkv, hdv, heads_per_block, has_sink, sink_score);                                            \
+                           H, Hkv, hdv, heads_per_block, has_sink, sink_score, bias_table, bias_len);                      \
     }
 #define AB_LAUNCH_NK(NK) AB_LAUNCH(NK, 1) AB_LAUNCH(NK, 2) AB_LAUNCH(NK, 3) AB_LAUNCH(NK, 4)
     AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(6) AB_LAUNCH_NK(8)

@@ -14,6 +14,8 @@
 // rotation, and that let a query attend to nothing:
 //  * slopes (fp32 [H]) with positions (int32 [n], the place of every query in its row): the score
 //    of query position i against key position j is lowered by slopes[h] * (i - j);
+//  * a distance table (fp32 [H, bias_len]) with positions: the score of query position i against key position j is
+//    raised by table[h, min(i - j, bias_len - 1)] (a learned bias per head and distance, constant from some distance on);
 //  * a sink: one more term exp(sink_score) in the softmax's denominator that carries no value
 //    (has_sink != 0). The running maximum and sum then start from that term instead of from nothing.
 #include "ka_common.h"
@@ -37,7 +39,8 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
                          const int* __restrict__ kv_lo, const int* __restrict__ kv_hi,
                          T* __restrict__ out, long out_row_stride, float scale, int H, int Hkv,
                          int hd, int hdv, int page_size, const int* __restrict__ positions,
-                         const float* __restrict__ slopes, int has_sink, float sink_score) {
+                         const float* __restrict__ slopes, int has_sink, float sink_score,
+                         const float* __restrict__ bias_table, int bias_len) {
     __shared__ float qs[ATT_MAX_HD];
     __shared__ float ps[KA_WAVE];
     __shared__ long offs[KA_WAVE];   // value cache offset of channel 0 of each key of the chunk
@@ -48,7 +51,8 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
     const T* qp = q + (size_t)t * q_row_stride + (size_t)h * hd;
     for (int d = lane; d < hd; d += KA_WAVE) qs[d] = ka_to_float(qp[d]) * scale;
     const float slope = slopes ? slopes[h] : 0.f;
-    const int place = slopes ? positions[t] : 0;
+    const int place = (slopes || bias_table) ? positions[t] : 0;
+    const float* bias_row = bias_table ? bias_table + (size_t)h * bias_len : nullptr;
     __syncthreads();
     const int* bt = block_table + (size_t)row * max_pages;
     const bool k_vectors = hd % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
@@ -79,6 +83,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
                 for (int d = 0; d < hd; ++d) acc = fmaf(qs[d], ka_to_float(kp[d]), acc);
             }
             s = slopes ? acc - slope * (float)(place - key) : acc;
+            if (bias_row) s += bias_row[min(max(place - key, 0), bias_len - 1)];
         }
         float m_new = fmaxf(m, ka_wave_max(s));
         float corr = expf(m - m_new);  // m = -inf at the first chunk gives 0
@@ -127,7 +132,9 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
                                 const int* token_row, const int* kv_lo, const int* kv_hi, void* out,
                                 long out_row_stride, float scale, int n, int H, int Hkv, int hd,
                                 int page_size, int hdv, const int* positions, const float* slopes,
-                                int has_sink, float sink_score, hipStream_t stream) {
+                                int has_sink, float sink_score, const float* bias_table, int bias_len,
+                                hipStream_t stream) {
+    KA_CHECK(bias_table == nullptr || (positions != nullptr && bias_len > 0), "ka_attention_generic: a distance table needs the queries' positions");
     KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0 && hdv > 0, "ka_attention_generic: bad sizes");
     KA_CHECK(hdv <= ATT_MAX_HD, "ka_attention_generic: value size %d above %d", hdv, ATT_MAX_HD);
     KA_CHECK(slopes == nullptr || positions != nullptr, "ka_attention_generic: slopes need the queries' positions");
@@ -141,12 +148,12 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_row_stride,
                            (const float*)k_cache, (const float*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (float*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score);
+                           sink_score, bias_table, bias_len);
     else if (dtype == KA_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
                            (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score);
+                           sink_score, bias_table, bias_len);
     else
         KA_CHECK(false, "ka_attention_generic: unsupported dtype %d", dtype);
     KA_LAUNCH_CHECK();

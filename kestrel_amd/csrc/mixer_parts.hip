@@ -1,0 +1,431 @@
+// Kernels of mixers that are more than "rotate, cache, attend": a root-mean-square norm, the preparation of
+// queries, keys and values of a step in one pass (norm with gains over a head or over the whole projection, a
+// rotation from frequencies, a factor on queries that grows with the place, values blended with those of another
+// layer, the paged cache write), an output gate, the sum of normalised branches, and a gated matrix memory
+// (a recurrent mixer with a state of fixed size per request). fp32 or bf16 storage, all arithmetic in fp32.
+#include "ka_common.h"
+
+constexpr int MP_THREADS = 256;
+constexpr int MP_WAVES = MP_THREADS / KA_WAVE;
+
+// Sum over the 256 threads of a workgroup, the same bits in every thread; `smem` holds MP_WAVES floats.
+__device__ __forceinline__ float mp_block_sum(float v, float* smem) {
+    v = ka_wave_sum(v);
+    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    __syncthreads();
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < MP_WAVES; ++w) total += smem[w];
+    return total;
+}
+
+__device__ __forceinline__ float mp_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+// ----------------------------------------------------------------------------
+// Root-mean-square norm: out = x / sqrt(mean(x^2) + eps) * gain over the last axis of fp32 rows (all, or
+// those that `rows` names).
+// ----------------------------------------------------------------------------
+template <typename TOut>
+__global__ void __launch_bounds__(MP_THREADS)
+rmsnorm_kernel(const float* __restrict__ x, const int* __restrict__ rows, const float* __restrict__ gain, float eps,
+               TOut* __restrict__ out, int dim) {
+    __shared__ float smem[MP_WAVES];
+    const int i = blockIdx.x;
+    const float* src = x + (size_t)(rows ? rows[i] : i) * dim;
+    TOut* dst = out + (size_t)i * dim;
+    float s = 0.f;
+    for (int d = threadIdx.x; d < dim; d += MP_THREADS) s += src[d] * src[d];
+    const float r = 1.0f / sqrtf(mp_block_sum(s, smem) / (float)dim + eps);
+    for (int d = threadIdx.x; d < dim; d += MP_THREADS) dst[d] = ka_from_float<TOut>(src[d] * r * (gain ? gain[d] : 1.f));
+}
+
+KA_API int ka_rmsnorm(const float* x, const int* rows, const float* gain, float eps, void* out, int out_dtype, int n,
+                      int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0 && eps >= 0.f, "ka_rmsnorm: bad sizes n=%d dim=%d", n, dim);
+    KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_rmsnorm: unsupported out dtype %d", out_dtype);
+    if (n == 0) return 0;
+    if (out_dtype == KA_F32)
+        hipLaunchKernelGGL(rmsnorm_kernel<float>, dim3(n), dim3(MP_THREADS), 0, stream, x, rows, gain, eps, (float*)out, dim);
+    else
+        hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, dim3(n), dim3(MP_THREADS), 0, stream, x, rows, gain, eps, (bf16_t*)out, dim);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Queries, keys and values of a step made ready for attention, a workgroup per token.
+// Row of `qkv`: [H hd queries | G hd keys | G hdv values]. In this order:
+//  * norm (norm_mode 1: every query and key head divided by its root mean square, gains [hd] shared by the
+//    heads; 2: all queries of the token by the root mean square over the whole H hd, likewise all keys, gains
+//    [H hd] and [G hd]; 0: none); gains optional;
+//  * rotation of the first `rot` channels of every head by the angles place * freqs[i], computed here in fp32
+//    (interleaved 1: channels 2i and 2i + 1 are a pair, 0: channels i and i + rot / 2); freqs null: none;
+//  * queries times 1 + q_coef * ln(floor((place + 1) / q_every) + 1) (q_every 0: no such factor);
+//  * values: blend 1 copies them to `v_other` (the values of this layer for later ones), blend 2 replaces them by
+//    (1 - lambda) v + lambda v_other with the fp32 scalar at `lambda`;
+//  * queries go back in place, keys in place and into the paged cache [pages, G, page_size, hd], values into
+//    [pages, G, hdv, page_size] (slots[t] = page * page_size + offset, negative or no slots: nothing is cached).
+// ----------------------------------------------------------------------------
+struct PrepareArgs {
+    void* qkv;
+    long row_stride;
+    const int* positions;
+    const int* slots;
+    void* k_cache;
+    void* v_cache;
+    int H, G, hd, hdv, page_size;
+    int norm_mode;
+    const float* q_gain;
+    const float* k_gain;
+    float eps;
+    const float* freqs;
+    int rot, interleaved;
+    float q_coef;
+    int q_every;
+    int blend;
+    void* v_other;
+    long v_other_stride;
+    const float* lambda;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(MP_THREADS) qkv_prepare_kernel(PrepareArgs a) {
+    extern __shared__ float sm[];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int heads = a.H + a.G, QK = heads * a.hd, half = a.rot / 2;
+    float* xs = sm;                    // the token's queries and keys as read
+    float* ss = xs + QK;               // sum of squares per head
+    float* cs = ss + heads;            // cosines, then sines, of the token's angles
+    float* sn = cs + half;
+    T* row = reinterpret_cast<T*>(a.qkv) + (size_t)t * a.row_stride;
+    const int pos = a.positions ? a.positions[t] : 0;
+    for (int e = tid; e < QK; e += MP_THREADS) xs[e] = ka_to_float(row[e]);
+    if (a.freqs)
+        for (int i = tid; i < half; i += MP_THREADS) sincosf((float)pos * a.freqs[i], &sn[i], &cs[i]);
+    __syncthreads();
+    if (a.norm_mode) {
+        const int wave = tid / KA_WAVE, lane = tid % KA_WAVE;
+        for (int h = wave; h < heads; h += MP_WAVES) {
+            float s = 0.f;
+            for (int c = lane; c < a.hd; c += KA_WAVE) s += xs[h * a.hd + c] * xs[h * a.hd + c];
+            s = ka_wave_sum(s);
+            if (lane == 0) ss[h] = s;
+        }
+        __syncthreads();
+    }
+    float r_all_q = 1.f, r_all_k = 1.f;
+    if (a.norm_mode == 2) {
+        float sq = 0.f, sk = 0.f;
+        for (int h = 0; h < a.H; ++h) sq += ss[h];
+        for (int h = a.H; h < heads; ++h) sk += ss[h];
+        r_all_q = 1.0f / sqrtf(sq / (float)(a.H * a.hd) + a.eps);
+        r_all_k = 1.0f / sqrtf(sk / (float)(a.G * a.hd) + a.eps);
+    }
+    const float q_factor = a.q_every > 0 ? 1.0f + a.q_coef * logf((float)((pos + 1) / a.q_every + 1)) : 1.0f;
+    const long slot = a.slots ? a.slots[t] : -1;
+    const long page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
+    T* k_cache = reinterpret_cast<T*>(a.k_cache);
+    T* v_cache = reinterpret_cast<T*>(a.v_cache);
+    for (int e = tid; e < QK; e += MP_THREADS) {
+        const int h = e / a.hd, c = e % a.hd;
+        const bool is_q = h < a.H;
+        float r = 1.f;
+        const float* gain = is_q ? a.q_gain : a.k_gain;
+        int gain_at = 0;                // index of channel 0 of this head in the gains
+        if (a.norm_mode == 1) r = 1.0f / sqrtf(ss[h] / (float)a.hd + a.eps);
+        else if (a.norm_mode == 2) {
+            r = is_q ? r_all_q : r_all_k;
+            gain_at = (is_q ? h : h - a.H) * a.hd;
+        }
+        const float own = xs[e] * r * (gain && a.norm_mode ? gain[gain_at + c] : 1.f);
+        float y = own;
+        if (a.freqs && c < a.rot) {
+            int i, partner;
+            bool first;
+            if (a.interleaved) { i = c >> 1; first = (c & 1) == 0; partner = c ^ 1; }
+            else { first = c < half; i = first ? c : c - half; partner = first ? c + half : c - half; }
+            const float other = xs[h * a.hd + partner] * r * (gain && a.norm_mode ? gain[gain_at + partner] : 1.f);
+            y = first ? own * cs[i] - other * sn[i] : own * cs[i] + other * sn[i];
+        }
+        if (is_q) {
+            row[e] = ka_from_float<T>(y * q_factor);
+        } else {
+            const T stored = ka_from_float<T>(y);
+            row[e] = stored;
+            if (slot >= 0) k_cache[(((size_t)page * a.G + (h - a.H)) * a.page_size + off) * a.hd + c] = stored;
+        }
+    }
+    T* vrow = row + QK;
+    const int VN = a.G * a.hdv;
+    const float lam = a.blend == 2 ? *a.lambda : 0.f;
+    T* other = a.blend ? reinterpret_cast<T*>(a.v_other) + (size_t)t * a.v_other_stride : nullptr;
+    for (int e = tid; e < VN; e += MP_THREADS) {
+        T v = vrow[e];
+        if (a.blend == 1) other[e] = v;
+        else if (a.blend == 2) {
+            v = ka_from_float<T>((1.0f - lam) * ka_to_float(v) + lam * ka_to_float(other[e]));
+            vrow[e] = v;
+        }
+        if (slot >= 0) {
+            const int g = e / a.hdv, c = e % a.hdv;
+            v_cache[(((size_t)page * a.G + g) * a.hdv + c) * a.page_size + off] = v;
+        }
+    }
+}
+
+KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* positions, const int* slots, void* k_cache,
+                          void* v_cache, int n, int H, int G, int hd, int hdv, int page_size, int norm_mode,
+                          const float* q_gain, const float* k_gain, float eps, const float* freqs, int rot, int interleaved,
+                          float q_coef, int q_every, int blend, void* v_other, long v_other_stride, const float* lambda,
+                          hipStream_t stream) {
+    const char* who = "ka_qkv_prepare";
+    KA_CHECK(n >= 0 && H > 0 && G > 0 && hd > 0 && hdv > 0 && page_size > 0, "%s: bad sizes", who);
+    KA_CHECK(row_stride >= (long)(H + G) * hd + (long)G * hdv, "%s: row stride %ld too small", who, row_stride);
+    KA_CHECK(norm_mode >= 0 && norm_mode <= 2 && eps >= 0.f, "%s: norm mode %d", who, norm_mode);
+    KA_CHECK(freqs == nullptr || (rot > 0 && rot <= hd && rot % 2 == 0), "%s: %d rotated channels of %d", who, rot, hd);
+    KA_CHECK(freqs == nullptr || positions != nullptr, "%s: a rotation needs the tokens' places", who);
+    KA_CHECK(q_every >= 0 && (q_every == 0 || positions != nullptr), "%s: the queries' factor needs the tokens' places", who);
+    KA_CHECK(interleaved == 0 || interleaved == 1, "%s: pairing must be 0 (halves) or 1 (interleaved)", who);
+    KA_CHECK(blend >= 0 && blend <= 2 && (blend == 0 || (v_other != nullptr && v_other_stride >= (long)G * hdv)),
+             "%s: blended values need the other layer's values", who);
+    KA_CHECK(blend != 2 || lambda != nullptr, "%s: a blend needs its weight", who);
+    KA_CHECK(slots == nullptr || (k_cache != nullptr && v_cache != nullptr), "%s: cache tensors missing", who);
+    KA_CHECK(dtype == KA_F32 || dtype == KA_BF16, "%s: unsupported dtype %d", who, dtype);
+    if (n == 0) return 0;
+    if (freqs == nullptr) rot = 0;
+    const size_t lds = ((size_t)(H + G) * hd + (H + G) + rot) * sizeof(float);
+    KA_CHECK(lds <= 64 * 1024, "%s: a token's queries and keys (%d values) do not fit in LDS", who, (H + G) * hd);
+    PrepareArgs a{qkv, row_stride, positions, slots, k_cache, v_cache, H, G, hd, hdv, page_size, norm_mode, q_gain, k_gain, eps,
+                  freqs, rot, interleaved, q_coef, q_every, blend, v_other, v_other_stride, lambda};
+    if (dtype == KA_F32) hipLaunchKernelGGL(qkv_prepare_kernel<float>, dim3(n), dim3(MP_THREADS), lds, stream, a);
+    else hipLaunchKernelGGL(qkv_prepare_kernel<bf16_t>, dim3(n), dim3(MP_THREADS), lds, stream, a);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Output gate: x[t, :] *= sigmoid(gate[t, :]) (both of the activation type, rows with strides of their own).
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(MP_THREADS)
+gate_mul_kernel(T* __restrict__ x, long x_stride, const T* __restrict__ gate, long gate_stride, int dim) {
+    T* xr = x + (size_t)blockIdx.x * x_stride;
+    const T* gr = gate + (size_t)blockIdx.x * gate_stride;
+    for (int d = threadIdx.x; d < dim; d += MP_THREADS) xr[d] = ka_from_float<T>(ka_to_float(xr[d]) * mp_sigmoid(ka_to_float(gr[d])));
+}
+
+KA_API int ka_gate_mul(void* x, long x_stride, const void* gate, long gate_stride, int dtype, int n, int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0 && x_stride >= dim && gate_stride >= dim, "ka_gate_mul: bad sizes");
+    KA_CHECK(dtype == KA_F32 || dtype == KA_BF16, "ka_gate_mul: unsupported dtype %d", dtype);
+    if (n == 0) return 0;
+    if (dtype == KA_F32)
+        hipLaunchKernelGGL(gate_mul_kernel<float>, dim3(n), dim3(MP_THREADS), 0, stream, (float*)x, x_stride, (const float*)gate, gate_stride, dim);
+    else
+        hipLaunchKernelGGL(gate_mul_kernel<bf16_t>, dim3(n), dim3(MP_THREADS), 0, stream, (bf16_t*)x, x_stride, (const bf16_t*)gate, gate_stride, dim);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// The sum of normalised branches into the stream: x += ca * rms(a) * gain_a [+ cb * rms(b) * gain_b], every
+// branch divided by its own root mean square over the row; all fp32.
+// ----------------------------------------------------------------------------
+__global__ void __launch_bounds__(MP_THREADS)
+branches_sum_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ gain_a, float ca,
+                    const float* __restrict__ b, const float* __restrict__ gain_b, float cb, float eps, int dim) {
+    __shared__ float smem[MP_WAVES];
+    const size_t at = (size_t)blockIdx.x * dim;
+    float sa = 0.f, sb = 0.f;
+    for (int d = threadIdx.x; d < dim; d += MP_THREADS) {
+        sa += a[at + d] * a[at + d];
+        if (b) sb += b[at + d] * b[at + d];
+    }
+    const float ra = 1.0f / sqrtf(mp_block_sum(sa, smem) / (float)dim + eps);
+    const float rb = b ? 1.0f / sqrtf(mp_block_sum(sb, smem) / (float)dim + eps) : 0.f;
+    for (int d = threadIdx.x; d < dim; d += MP_THREADS) {
+        float y = ca * (a[at + d] * ra * (gain_a ? gain_a[d] : 1.f));
+        if (b) y += cb * (b[at + d] * rb * (gain_b ? gain_b[d] : 1.f));
+        x[at + d] += y;
+    }
+}
+
+KA_API int ka_branches_sum(float* x, const float* a, const float* gain_a, float ca, const float* b, const float* gain_b,
+                           float cb, float eps, int n, int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0 && eps >= 0.f && a != nullptr, "ka_branches_sum: bad sizes");
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(branches_sum_kernel, dim3(n), dim3(MP_THREADS), 0, stream, x, a, gain_a, ca, b, gain_b, cb, eps, dim);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Gated matrix memory: per request and head a state S [d, dv], n [d] and a running maximum m (fp32, in that
+// order in `state`, [state rows, heads, d dv + d + 1]), advanced token by token:
+//     li = cap tanh(gi / cap),  lf = logsigmoid(cap tanh(gf / cap))          (gi, gf: pre[t, head], pre[t, heads + head])
+//     m' = max(lf + m, li);  S' = e^(lf + m - m') S + e^(li - m') k v^T;  n' likewise with k
+//     o = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6),  q already times q_scale
+//     out[t, head dv + j] = o_j / sqrt(mean_j(o^2) + eps) * gain[head dv + j] * sigmoid(gate[t, head dv + j])
+// A workgroup per (head, row) walks over the row's tokens (cu_q) in order. The state lives in LDS while it does
+// (LDS_STATE) or stays in memory (rows of one token, states too large for LDS). A row without a request
+// (row_slot < 0) writes zeros and touches no state.
+// ----------------------------------------------------------------------------
+struct MemoryArgs {
+    const void* q; const void* k; const void* v; const void* gate;     // rows of the activation type, one stride
+    long stride;
+    const float* pre;              // fp32 [n, 2 heads]
+    float* state;
+    const int* cu_q;
+    const int* row_slot;
+    const float* gain;             // fp32 [heads dv] or null
+    void* out;
+    long out_stride;
+    int heads, d, dv, parts;
+    float q_scale, cap, eps;
+};
+
+template <typename T, bool LDS_STATE>
+__global__ void __launch_bounds__(MP_THREADS) matrix_memory_kernel(MemoryArgs a) {
+    extern __shared__ float sm[];
+    const int head = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+    const int t0 = a.cu_q[r], t1 = a.cu_q[r + 1];
+    if (t0 >= t1) return;
+    const int d = a.d, dv = a.dv, parts = a.parts;
+    T* out = reinterpret_cast<T*>(a.out);
+    const int slot = a.row_slot[r];
+    if (slot < 0) {
+        for (int t = t0; t < t1; ++t)
+            for (int j = tid; j < dv; j += MP_THREADS) out[(size_t)t * a.out_stride + head * dv + j] = ka_from_float<T>(0.f);
+        return;
+    }
+    const int per_head = d * dv + d + 1;
+    float* st = a.state + ((size_t)slot * a.heads + head) * per_head;
+    float* S = LDS_STATE ? sm : st;
+    float* nv = S + d * dv;
+    float* qs = sm + (LDS_STATE ? d * dv + d : 0);
+    float* ks = qs + d;
+    float* vs = ks + d;
+    float* part = vs + dv;             // [parts, dv]
+    float* red = part + parts * dv;    // [1 + MP_WAVES]
+    if (LDS_STATE)
+        for (int e = tid; e < d * dv + d; e += MP_THREADS) sm[e] = st[e];
+    float m = st[d * dv + d];
+    const T* qp = reinterpret_cast<const T*>(a.q);
+    const T* kp = reinterpret_cast<const T*>(a.k);
+    const T* vp = reinterpret_cast<const T*>(a.v);
+    const T* gp = reinterpret_cast<const T*>(a.gate);
+    for (int t = t0; t < t1; ++t) {
+        const size_t at = (size_t)t * a.stride;
+        __syncthreads();               // (the token before is done with qs, ks, vs, part and red)
+        for (int e = tid; e < d; e += MP_THREADS) {
+            qs[e] = ka_to_float(qp[at + head * d + e]) * a.q_scale;
+            ks[e] = ka_to_float(kp[at + head * d + e]);
+        }
+        for (int j = tid; j < dv; j += MP_THREADS) vs[j] = ka_to_float(vp[at + head * dv + j]);
+        const float gi = a.pre[(size_t)t * 2 * a.heads + head], gf = a.pre[(size_t)t * 2 * a.heads + a.heads + head];
+        const float li = a.cap * tanhf(gi / a.cap);
+        const float z = a.cap * tanhf(gf / a.cap);
+        const float lf = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+        const float m_new = fmaxf(lf + m, li);
+        const float keep = expf(lf + m - m_new), take = expf(li - m_new);
+        m = m_new;
+        __syncthreads();
+        if (tid < KA_WAVE) {
+            float acc = 0.f;
+            for (int e = tid; e < d; e += KA_WAVE) {
+                const float x = keep * nv[e] + take * ks[e];
+                nv[e] = x;
+                acc += x * qs[e];
+            }
+            acc = ka_wave_sum(acc);
+            if (tid == 0) red[0] = acc;
+        }
+        for (int idx = tid; idx < parts * dv; idx += MP_THREADS) {
+            const int j = idx % dv, p = idx / dv;
+            const float vj = take * vs[j];
+            float acc = 0.f;
+            for (int i = p; i < d; i += parts) {
+                const float s = keep * S[(size_t)i * dv + j] + ks[i] * vj;
+                S[(size_t)i * dv + j] = s;
+                acc += s * qs[i];
+            }
+            part[idx] = acc;
+        }
+        __syncthreads();
+        const float den = fmaxf(fabsf(red[0]), expf(-m_new)) + 1e-6f;
+        float o[4];                    // (dv <= 4 * 256)
+        float sq = 0.f;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = tid + u * MP_THREADS;
+            o[u] = 0.f;
+            if (j < dv) {
+                float acc = 0.f;
+                for (int p = 0; p < parts; ++p) acc += part[p * dv + j];
+                o[u] = acc / den;
+                sq += o[u] * o[u];
+            }
+        }
+        const float rr = 1.0f / sqrtf(mp_block_sum(sq, red + 1) / (float)dv + a.eps);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int j = tid + u * MP_THREADS;
+            if (j < dv) {
+                const int c = head * dv + j;
+                const float g = gp ? mp_sigmoid(ka_to_float(gp[at + c])) : 1.f;
+                out[(size_t)t * a.out_stride + c] = ka_from_float<T>(o[u] * rr * (a.gain ? a.gain[c] : 1.f) * g);
+            }
+        }
+    }
+    __syncthreads();
+    if (LDS_STATE)
+        for (int e = tid; e < d * dv + d; e += MP_THREADS) st[e] = sm[e];
+    if (tid == 0) st[d * dv + d] = m;
+}
+
+// Floats of LDS that the kernel needs beside the state.
+static size_t mm_scratch_floats(int d, int dv, int parts) { return (size_t)2 * d + dv + (size_t)parts * dv + 1 + MP_WAVES; }
+
+constexpr size_t MM_LDS_LIMIT = 128 * 1024;
+
+KA_API int ka_matrix_memory(const void* q, const void* k, const void* v, const void* gate, long stride, int dtype,
+                            const float* pre, float* state, int state_rows, const int* cu_q, const int* row_slot,
+                            const float* gain, void* out, long out_stride, int n_rows, int heads, int d, int dv,
+                            float q_scale, float cap, float eps, int single_tokens, hipStream_t stream) {
+    const char* who = "ka_matrix_memory";
+    KA_CHECK(n_rows >= 0 && heads > 0 && d > 0 && dv > 0 && state_rows > 0, "%s: bad sizes", who);
+    KA_CHECK(dv <= 4 * MP_THREADS, "%s: value size %d above %d", who, dv, 4 * MP_THREADS);
+    KA_CHECK(cap > 0.f && eps >= 0.f, "%s: the gates' cap must be positive", who);
+    KA_CHECK(dtype == KA_F32 || dtype == KA_BF16, "%s: unsupported dtype %d", who, dtype);
+    KA_CHECK(heads <= 65535 && n_rows <= 65535, "%s: too many heads or rows", who);
+    if (n_rows == 0) return 0;
+    int parts = MP_THREADS / dv;
+    parts = parts < 1 ? 1 : (parts > d ? d : parts);
+    const size_t scratch = mm_scratch_floats(d, dv, parts) * sizeof(float);
+    const size_t with_state = scratch + ((size_t)d * dv + d) * sizeof(float);
+    // rows of one token read and write every number of the state once either way: no detour through LDS
+    const bool in_lds = !single_tokens && with_state <= MM_LDS_LIMIT;
+    KA_CHECK(scratch <= MM_LDS_LIMIT, "%s: heads of %d x %d do not fit", who, d, dv);
+    MemoryArgs a{q, k, v, gate, stride, pre, state, cu_q, row_slot, gain, out, out_stride, heads, d, dv, parts, q_scale, cap, eps};
+    const dim3 grid(heads, n_rows), block(MP_THREADS);
+#define MM_LAUNCH(T, IN_LDS, BYTES)                                                                                        \
+    do {                                                                                                                   \
+        static bool sized = false;                                                                                         \
+        if (!sized) {                                                                                                      \
+            (void)hipFuncSetAttribute((const void*)matrix_memory_kernel<T, IN_LDS>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)MM_LDS_LIMIT); \
+            sized = true;                                                                                                  \
+        }                                                                                                                  \
+        hipLaunchKernelGGL((matrix_memory_kernel<T, IN_LDS>), grid, block, BYTES, stream, a);                              \
+    } while (0)
+    if (dtype == KA_F32) {
+        if (in_lds) MM_LAUNCH(float, true, with_state);
+        else MM_LAUNCH(float, false, scratch);
+    } else {
+        if (in_lds) MM_LAUNCH(bf16_t, true, with_state);
+        else MM_LAUNCH(bf16_t, false, scratch);
+    }
+#undef MM_LAUNCH
+    KA_LAUNCH_CHECK();
+    return 0;
+}

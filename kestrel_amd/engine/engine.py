@@ -192,7 +192,8 @@ class InferenceEngine:
         free_bytes, _total = torch.cuda.mem_get_info(device)
         n_pages = pool_pages(cfg, sizing.bytes_per_page(), max_seq, free_bytes)
         self.runner = make_runner(net, cfg.page_size, n_pages, cfg.max_batch_size,
-                                  max_tokens_per_step=cfg.max_num_batched_tokens, enable_graphs=cfg.enable_graphs)
+                                  max_tokens_per_step=cfg.max_num_batched_tokens, enable_graphs=cfg.enable_graphs,
+                                  max_positions=max_seq)
         _LOGGER.info("cache pool: %d pages of %d tokens per group of layers (%.2f GiB), %d request slots, contexts up to %d",
                      n_pages, cfg.page_size, n_pages * sizing.bytes_per_page() / float(1 << 30), cfg.max_batch_size, max_seq)
         sampler = Sampler(device, cfg.seed, pending=self.runner.pending)

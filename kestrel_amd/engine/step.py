@@ -31,7 +31,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..cache.manager import CacheManager
+from ..cache.manager import CacheManager, reach
 from ..models.decoder import DecoderModel
 from .batch import GroupBatch, StepBatch, Workspace
 
@@ -210,8 +210,13 @@ class ModelRunner:
 
     def __init__(self, model: DecoderModel, cache: CacheManager, device: torch.device,
                  max_tokens_per_step: int = 4096, enable_graphs: bool = False,
-                 max_graph_batch: Optional[int] = None) -> None:
+                 max_graph_batch: Optional[int] = None, max_positions: Optional[int] = None) -> None:
         self.model, self.cache, self.device = model, cache, device
+        # the longest sequence a request may grow to: what the model allows (a design without a bound of its own names
+        # a very large number) and what the caller allows; a row can never hold more than the pool does, which bounds
+        # the width of block tables and the longest row that graphs are captured for
+        self.max_positions = min(int(model.plan.max_positions), int(max_positions or model.plan.max_positions))
+        self._longest_row = min(self.max_positions, cache.n_pages * cache.page_size)
         self.max_tokens_per_step = max_tokens_per_step
         self.workspace = Workspace(device)
         self.layer_caches = cache.layer_caches()
@@ -223,7 +228,7 @@ class ModelRunner:
         self.enable_graphs = enable_graphs
         self._buckets = graph_buckets(min(max_graph_batch or cache.max_requests, cache.max_requests))
         self._graphs: Dict[int, _GraphState] = {}
-        self._pages_cap = -(-model.plan.max_positions // cache.page_size)
+        self._pages_cap = -(-self._longest_row // cache.page_size)
         self.graph_replays = 0
         # steps of any shape (prompt portions, beside decoded tokens or not) are replayed too, if every
         # part of the model can be (``Part.replays_every_step``): per bucket of tokens and of rows
@@ -290,8 +295,8 @@ class ModelRunner:
             start = self.held[e.slot] if e.start is None else int(e.start)
             if start != self.held[e.slot]:
                 raise refuse(f"portion starts at {start} but the request holds {self.held[e.slot]} tokens")
-            if start + q > plan.max_positions:
-                raise refuse(f"{start + q} tokens exceed the model's {plan.max_positions} positions")
+            if start + q > self.max_positions:
+                raise refuse(f"{start + q} tokens exceed the {self.max_positions} positions a request may hold")
             if q <= self.SCALAR_ROW:
                 n_given = 0
                 for tok in e.tokens:
@@ -375,7 +380,7 @@ class ModelRunner:
         cu_q = [0]
         kv_len: List[int] = []
         slots = [_Column() for _ in range(n_groups)]
-        kv_lo = [_Column() if g.spec.window is not None else None for g in cache.groups]
+        kv_lo = [_Column() if reach(g.spec) is not None else None for g in cache.groups]
         max_pages = max(1, fixed_pages)
         max_q = max_kv = 1
         causal_only = True
@@ -628,7 +633,7 @@ class ModelRunner:
                                      workspace=state.workspace)
             # the decode attention kernel cuts a row's keys by the longest context of the batch: a
             # graph must cut the same way on every replay, so it is captured for the longest possible
-            blank.max_kv = self.model.plan.max_positions
+            blank.max_kv = self._longest_row
             self._run_aside(blank)
             state.workspace.freeze()
             graph = torch.cuda.CUDAGraph()
@@ -655,7 +660,7 @@ class ModelRunner:
         """A step of the layout ``(tokens, rows)`` whose tokens belong to no request."""
         blank = self.build_batch([], pad_rows=rows, pad_tokens=tokens, fixed_pages=self._pages_cap, meta=meta,
                                  workspace=workspace or self._mixed_workspace)
-        blank.max_kv = self.model.plan.max_positions       # (kernels that size themselves by the longest row)
+        blank.max_kv = self._longest_row       # (kernels that size themselves by the longest row)
         blank.given_embeds = self._mixed_given[:tokens]
         return blank
 
@@ -789,7 +794,7 @@ class ModelRunner:
             done["capture_s"] = time.perf_counter() - started
         # prompts: the largest first (every scratch tensor at its largest), then one per bucket of rows of
         # the vendor library's plans, the smallest (64 tokens: the kernels of few rows) last
-        fits = min(limit, plan.max_positions - 1, min(g.pool.free_count for g in cache.groups) * cache.page_size
+        fits = min(limit, self.max_positions - 1, min(g.pool.free_count for g in cache.groups) * cache.page_size
                    if cache.groups else limit)
         sizes = sorted({fits} | set(range(64, fits, 64)), reverse=True) if fits >= 1 else []
         if self.model.dtype != torch.bfloat16:

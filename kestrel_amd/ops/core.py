@@ -31,7 +31,17 @@ _SIGNATURES = {
                           _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                              _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
-                             _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p],
+                             _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_int, _c_void_p],
+    "ka_rmsnorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_qkv_prepare": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
+                       _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_float, _c_int,
+                       _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p],
+    "ka_gate_mul": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_branches_sum": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_float, _c_float, _c_int, _c_int,
+                        _c_void_p],
+    "ka_matrix_memory": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                         _c_void_p, _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
+                         _c_int, _c_void_p],
     "ka_add_table_rows": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_cast_columns": [_c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],
     "ka_add_scaled": [_c_void_p, _c_void_p, _c_float, _c_long, _c_void_p],
@@ -319,6 +329,128 @@ def unit_norm_cache(qkv: torch.Tensor, slots: Optional[torch.Tensor], k_cache: O
 ROTARY_PAIRINGS = {"halves": 0, "interleaved": 1}
 
 
+def rmsnorm(x: torch.Tensor, gain: Optional[torch.Tensor], eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+    """``out = x / sqrt(mean(x^2) + eps) * gain`` over the last axis of fp32 rows of ``x`` (all, or those named by ``rows``)."""
+    _dev(x, gain, out, rows)
+    n, dim = out.shape
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.shape[1] == dim and x.is_contiguous(), "rmsnorm: x must be contiguous fp32 [*, dim]")
+    _need(gain is None or (gain.dtype == torch.float32 and gain.numel() == dim), "rmsnorm: gain must be fp32 [dim]")
+    _need(out.is_contiguous(), "rmsnorm: out must be contiguous")
+    if rows is None:
+        _need(x.shape[0] == n, "rmsnorm: row counts differ")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() == n and rows.is_contiguous(), "rmsnorm: rows int32 [n]")
+    _check(lib().ka_rmsnorm(x.data_ptr(), _ptr(rows), _ptr(gain), float(eps), out.data_ptr(), code_of(out.dtype), n, dim, stream_ptr()))
+
+
+QK_NORM_SCOPES = {None: 0, "head": 1, "projection": 2}
+VALUE_BLENDS = {None: 0, "source": 1, "blend": 2}
+
+
+def qkv_prepare(qkv: torch.Tensor, positions: Optional[torch.Tensor], slots: Optional[torch.Tensor], k_cache: Optional[torch.Tensor],
+                v_cache: Optional[torch.Tensor], n_heads: int, n_kv_heads: int, head_dim: int, value_dim: int, page_size: int,
+                norm_scope: Optional[str] = None, q_gain: Optional[torch.Tensor] = None, k_gain: Optional[torch.Tensor] = None,
+                eps: float = 0.0, freqs: Optional[torch.Tensor] = None, pairing: str = "halves", q_growth=None,
+                blend: Optional[str] = None, v_other: Optional[torch.Tensor] = None, blend_weight: Optional[torch.Tensor] = None) -> None:
+    """Queries, keys and values of a step made ready for attention in one pass over ``qkv`` ``[n, H hd | Hkv hd | Hkv hdv]``
+    (rows may lie in a wider buffer): the norm of queries and keys (``norm_scope`` ``"head"``: every head by its own root mean
+    square, gains ``[hd]``; ``"projection"``: all queries of a token by one, all keys by one, gains ``[H hd]`` and ``[Hkv hd]``),
+    then the rotation of the first ``2 len(freqs)`` channels of every head by ``place * freqs`` (fp32 ``freqs``; ``pairing`` as
+    in ``rope_cache``), then queries times ``1 + coef * ln(floor((place + 1) / every) + 1)`` for ``q_growth = (coef, every)``;
+    values copied to ``v_other`` (``blend`` ``"source"``) or replaced by ``(1 - w) v + w v_other`` (``"blend"``, ``w`` the fp32
+    scalar tensor ``blend_weight``); queries and keys back in place, keys and values into the paged cache at ``slots``."""
+    _need(pairing in ROTARY_PAIRINGS, f"qkv_prepare: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
+    _need(norm_scope in QK_NORM_SCOPES and blend in VALUE_BLENDS, "qkv_prepare: unknown norm scope or blend")
+    _dev(qkv, positions, slots, k_cache, v_cache, q_gain, k_gain, freqs, v_other, blend_weight)
+    n = qkv.shape[0]
+    total = (n_heads + n_kv_heads) * head_dim + n_kv_heads * value_dim
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == total, "qkv_prepare: qkv must be [n, H hd + Hkv hd + Hkv hdv]")
+    for t in (positions, slots):
+        _need(t is None or (t.dtype == torch.int32 and t.numel() == n and t.is_contiguous()), "qkv_prepare: per-token int32 [n] expected")
+    if slots is not None:
+        _need(k_cache is not None and v_cache is not None, "qkv_prepare: cache tensors missing")
+        _check_caches("qkv_prepare", k_cache, v_cache, qkv.dtype, n_kv_heads, page_size, head_dim, value_dim)
+    per_head = norm_scope == "head"
+    for gain, heads in ((q_gain, n_heads), (k_gain, n_kv_heads)):
+        _need(gain is None or (gain.dtype == torch.float32 and gain.is_contiguous()
+                               and gain.numel() == (head_dim if per_head else heads * head_dim)), "qkv_prepare: gains fp32 [hd] or [heads hd]")
+    rot = 0
+    if freqs is not None:
+        _need(freqs.dtype == torch.float32 and freqs.dim() == 1 and freqs.is_contiguous(), "qkv_prepare: freqs fp32 [R / 2]")
+        rot = 2 * freqs.numel()
+    coef, every = (float(q_growth[0]), int(q_growth[1])) if q_growth is not None else (0.0, 0)
+    _need(q_growth is None or every > 0, "qkv_prepare: the queries' factor needs a positive period")
+    if blend is not None:
+        _need(v_other is not None and v_other.dtype == qkv.dtype and v_other.dim() == 2 and v_other.stride(1) == 1
+              and tuple(v_other.shape) == (n, n_kv_heads * value_dim), "qkv_prepare: v_other must be [n, Hkv hdv] of the qkv type")
+        _need(blend != "blend" or (blend_weight is not None and blend_weight.dtype == torch.float32 and blend_weight.numel() == 1),
+              "qkv_prepare: the blend's weight must be one fp32 number")
+    _check(lib().ka_qkv_prepare(qkv.data_ptr(), code_of(qkv.dtype), qkv.stride(0) if n > 1 else max(qkv.stride(0), total), _ptr(positions), _ptr(slots),
+                                _ptr(k_cache), _ptr(v_cache), n, n_heads, n_kv_heads, head_dim, value_dim, page_size,
+                                QK_NORM_SCOPES[norm_scope], _ptr(q_gain), _ptr(k_gain), float(eps), _ptr(freqs), rot,
+                                ROTARY_PAIRINGS[pairing], coef, every, VALUE_BLENDS[blend], _ptr(v_other),
+                                (v_other.stride(0) if n > 1 else n_kv_heads * value_dim) if v_other is not None else 0, _ptr(blend_weight), stream_ptr()))
+
+
+def gate_mul(x: torch.Tensor, gate: torch.Tensor) -> None:
+    """``x *= sigmoid(gate)`` element by element; both ``[n, dim]`` of one type, rows may lie in wider buffers."""
+    _dev(x, gate)
+    n, dim = x.shape
+    _need(gate.shape == x.shape and gate.dtype == x.dtype and x.stride(1) == 1 and gate.stride(1) == 1, "gate_mul: two [n, dim] of one type")
+    _check(lib().ka_gate_mul(x.data_ptr(), x.stride(0) if n > 1 else dim, gate.data_ptr(), gate.stride(0) if n > 1 else dim,
+                             code_of(x.dtype), n, dim, stream_ptr()))
+
+
+def branches_sum(x: torch.Tensor, a: torch.Tensor, gain_a: Optional[torch.Tensor], weight_a: float,
+                 b: Optional[torch.Tensor] = None, gain_b: Optional[torch.Tensor] = None, weight_b: float = 0.0, eps: float = 0.0) -> None:
+    """``x += weight_a * rms(a) * gain_a + weight_b * rms(b) * gain_b``: every branch divided by its own root mean square
+    ``sqrt(mean(square) + eps)`` over the row; all contiguous fp32 ``[n, dim]``, gains fp32 ``[dim]``."""
+    _dev(x, a, gain_a, b, gain_b)
+    n, dim = x.shape
+    for t in (x, a, b):
+        _need(t is None or (t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == (n, dim)), "branches_sum: contiguous fp32 [n, dim]")
+    for g in (gain_a, gain_b):
+        _need(g is None or (g.dtype == torch.float32 and g.numel() == dim and g.is_contiguous()), "branches_sum: gains fp32 [dim]")
+    _check(lib().ka_branches_sum(x.data_ptr(), a.data_ptr(), _ptr(gain_a), float(weight_a), _ptr(b), _ptr(gain_b), float(weight_b),
+                                 float(eps), n, dim, stream_ptr()))
+
+
+def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
+                  row_slot: torch.Tensor, gain: Optional[torch.Tensor], out: torch.Tensor, n_heads: int, head_dim: int,
+                  value_dim: int, q_scale: float, cap: float, eps: float, single_tokens: bool) -> None:
+    """The gated matrix memory over the packed tokens of a step. ``projected`` ``[n, *]`` holds queries, keys, values and
+    (optionally) the output gate's pre-activations at the column ``offsets = (q, k, v, gate or None)``; ``pre`` fp32
+    ``[n, 2 heads]`` the pre-activations of the input gates, then of the forget gates; ``state`` fp32
+    ``[slots + 1, heads * (hd * hdv + hd + 1)]`` (per head the matrix, the normaliser and the running maximum), advanced in
+    place for row ``r`` at ``row_slot[r]`` over its tokens ``cu_q[r] .. cu_q[r + 1]`` (a negative slot: zeros are written,
+    no state is touched). ``out`` ``[n, heads * hdv]``: every head's read-out divided by its root mean square, times ``gain``
+    (fp32 ``[heads * hdv]``), times the sigmoid of the gate."""
+    _dev(projected, pre, state, cu_q, row_slot, gain, out)
+    n = projected.shape[0]
+    n_rows = row_slot.numel()
+    oq, ok, ov, og = offsets
+    width = projected.shape[1]
+    _need(projected.dim() == 2 and projected.stride(1) == 1, "matrix_memory: projected rows must be contiguous")
+    _need(max(oq, ok) + n_heads * head_dim <= width and ov + n_heads * value_dim <= width
+          and (og is None or og + n_heads * value_dim <= width), "matrix_memory: offsets outside the projected rows")
+    _need(pre.dtype == torch.float32 and pre.is_contiguous() and tuple(pre.shape) == (n, 2 * n_heads), "matrix_memory: pre fp32 [n, 2 heads]")
+    per_head = head_dim * value_dim + head_dim + 1
+    _need(state.dtype == torch.float32 and state.is_contiguous() and state.dim() == 2 and state.shape[1] == n_heads * per_head,
+          "matrix_memory: state fp32 [slots, heads * (hd * hdv + hd + 1)]")
+    _need(cu_q.dtype == torch.int32 and cu_q.numel() == n_rows + 1 and row_slot.dtype == torch.int32, "matrix_memory: cu_q int32 [rows + 1]")
+    _need(out.dtype == projected.dtype and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * value_dim),
+          "matrix_memory: out must be [n, heads hdv] of the projected type")
+    _need(gain is None or (gain.dtype == torch.float32 and gain.numel() == n_heads * value_dim), "matrix_memory: gain fp32 [heads hdv]")
+    size = projected.element_size()
+    base = projected.data_ptr()
+    stride = projected.stride(0) if n > 1 else width
+    _check(lib().ka_matrix_memory(base + oq * size, base + ok * size, base + ov * size, None if og is None else base + og * size,
+                                  stride, code_of(projected.dtype), pre.data_ptr(), state.data_ptr(), state.shape[0],
+                                  cu_q.data_ptr(), row_slot.data_ptr(), _ptr(gain), out.data_ptr(),
+                                  out.stride(0) if n > 1 else n_heads * value_dim, n_rows, n_heads, head_dim, value_dim,
+                                  float(q_scale), float(cap), float(eps), int(bool(single_tokens)), stream_ptr()))
+
+
 def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
                table: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, pairing: str = "halves") -> None:
@@ -374,14 +506,16 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       token_row: torch.Tensor, kv_lo: Optional[torch.Tensor], kv_hi: torch.Tensor,
                       out: torch.Tensor, scale: float, n_heads: int, n_kv_heads: int, head_dim: int,
                       value_dim: Optional[int] = None, positions: Optional[torch.Tensor] = None,
-                      slopes: Optional[torch.Tensor] = None, sink: Optional[float] = None) -> None:
+                      slopes: Optional[torch.Tensor] = None, sink: Optional[float] = None,
+                      bias_table: Optional[torch.Tensor] = None) -> None:
     """Paged attention of ``n`` packed tokens; ``q`` may be a strided view into a qkv buffer.
 
     ``value_dim``: size of a value head where it differs from ``head_dim`` (``out`` is ``[n, H value_dim]``).
     ``slopes`` (fp32 ``[H]``) with ``positions`` (int32 ``[n]``): the score of a query at place ``i`` against the key
     at place ``j`` is lowered by ``slopes[h] * (i - j)``. ``sink``: the score of one more term of the softmax's
-    denominator that carries no value (``None``: no such term)."""
-    _dev(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, positions, slopes)
+    denominator that carries no value (``None``: no such term). ``bias_table`` (fp32 ``[H, T]``) with ``positions``: the
+    score is raised by ``bias_table[h, min(i - j, T - 1)]``."""
+    _dev(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, positions, slopes, bias_table)
     n = q.shape[0]
     value_dim = head_dim if value_dim is None else int(value_dim)
     _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * head_dim, "attention: q must be [n, >= H hd]")
@@ -394,6 +528,11 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
               "attention: slopes must be fp32 [H]")
         _need(positions is not None and positions.dtype == torch.int32 and positions.numel() == n and positions.is_contiguous(),
               "attention: slopes need the queries' positions, int32 [n]")
+    if bias_table is not None:
+        _need(bias_table.dtype == torch.float32 and bias_table.dim() == 2 and bias_table.shape[0] == n_heads
+              and bias_table.is_contiguous(), "attention: the distance table must be contiguous fp32 [H, T]")
+        _need(positions is not None and positions.dtype == torch.int32 and positions.numel() == n and positions.is_contiguous(),
+              "attention: a distance table needs the queries' positions, int32 [n]")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "attention: block table must be contiguous int32 [rows, pages]")
     for t in (token_row, kv_hi) + ((kv_lo,) if kv_lo is not None else ()):
@@ -402,8 +541,9 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                                       v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
                                       token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
                                       out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size,
-                                      value_dim, _ptr(positions) if slopes is not None else None, _ptr(slopes),
-                                      int(sink is not None), float(sink or 0.0), stream_ptr()))
+                                      value_dim, _ptr(positions) if (slopes is not None or bias_table is not None) else None,
+                                      _ptr(slopes), int(sink is not None), float(sink or 0.0), _ptr(bias_table),
+                                      int(bias_table.shape[1]) if bias_table is not None else 0, stream_ptr()))
 
 
 def _pending_args(who: str, rows: int, pending, pending_at):

@@ -54,7 +54,7 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],      # W, ldw, bias, out, ..., stream
     "ka_attention_biased_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
-                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p],
     "ka_linear_skinny_norm_store": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p,
                                     _c_int, _c_long, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
 }
@@ -598,7 +598,7 @@ def biased_query_block(head_dim: int, value_dim: int) -> Optional[int]:
 
 
 def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
-                          head_dim, value_dim, positions, slopes, sink, batch) -> bool:
+                          head_dim, value_dim, positions, slopes, sink, batch, bias_table=None) -> bool:
     """Attention with the further terms of ``ops.core.attention_generic`` (values of ``value_dim`` channels, ``slopes``
     times the distance taken off the scores, a ``sink`` in the softmax's denominator) on the matrix cores, for prompt
     portions, mixed steps and decode steps alike. False: not covered (head sizes, page size, alignment, no list of
@@ -615,6 +615,9 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         return False
     if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or positions is None):
         raise KernelError("attention: slopes must be fp32 [H] and come with the queries' positions")
+    if bias_table is not None and (bias_table.dtype != torch.float32 or bias_table.dim() != 2 or bias_table.shape[0] != n_heads
+                                   or not bias_table.is_contiguous() or positions is None):
+        raise KernelError("attention: the distance table must be contiguous fp32 [H, T] and come with the queries' positions")
     if batch.decode_only:
         rows = first = None
         n_blocks = 0
@@ -637,5 +640,6 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
         _ptr(rows), _ptr(first), n_blocks, batch.cu_q.data_ptr(), token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(),
         _ptr(positions), _ptr(slopes), out.data_ptr(), out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim,
-        value_dim, page_size, waves, int(sink is not None), float(sink or 0.0), stream_ptr()))
+        value_dim, page_size, waves, int(sink is not None), float(sink or 0.0), _ptr(bias_table),
+        int(bias_table.shape[1]) if bias_table is not None else 0, stream_ptr()))
     return True

@@ -37,6 +37,17 @@ class PagedAttention(Mixer):
     nothing; the three projections stored as three tensors (``split_projections``). With any of the middle four
     the mixer takes no rotation, and runs through kernels of its own (``ops.core.unit_norm_cache`` and the
     attention kernels that know these terms).
+
+    A third family of forms is made ready by one kernel (``ops.core.qkv_prepare``: norm, rotation, factor, blend and cache
+    write in one pass over the projected rows), again each by its field and in any combination: queries and keys
+    normalised with learned gains over a head or over the whole projection (``qk_norm``); a rotation given by
+    frequencies, with either pairing of channels (a position encoding that offers ``Rotation.frequencies``); queries
+    times a factor that grows with the place (``query_growth``); a learned bias per bucket of distance and head
+    (``distance_buckets``, tensor ``rel``, turned into a table by distance when the weights are bound); values blended
+    with those of another layer of the same step (``value_blend``, tensor ``vmix``); the heads multiplied by the sigmoid
+    of a further projection of the input before the output projection (``output_gate``, tensor ``gate.weight``, which
+    rides in the launch of the q|k|v projection). ``chunk`` is a mask like ``window``: it only changes which keys a
+    token reads (``kv_lo``) and which pages go back.
     """
 
     replays_every_step = True
@@ -57,9 +68,24 @@ class PagedAttention(Mixer):
         self.sink = getattr(spec, "sink", None)
         self.distance = getattr(spec, "distance_slopes", None)
         # the forms that the kernels of the rotary path know nothing of
+        self.qk_norm = getattr(spec, "qk_norm", None)
+        self.growth = getattr(spec, "query_growth", None)
+        self.buckets = getattr(spec, "distance_buckets", None)
+        self.blend = getattr(spec, "value_blend", None)
+        self.gated = bool(getattr(spec, "output_gate", False))
+        if self.qk_norm is not None and (self.qk_norm.scope not in ("head", "projection") or self.unit_norm_eps is not None):
+            raise ValueError("qk_norm takes the scope 'head' or 'projection' and stands instead of qk_unit_norm_eps")
+        if self.blend is not None and self.blend.role not in ("source", "blend"):
+            raise ValueError(f"a value blend has the role 'source' or 'blend', got {self.blend.role!r}")
         self.extended = self.value_dim != spec.head_dim or self.unit_norm_eps is not None or self.sink is not None \
-            or self.distance is not None
+            or self.distance is not None or self.buckets is not None
+        # the forms that ``ops.core.qkv_prepare`` makes ready (a rotation by frequencies, found when the weights are bound, too)
+        self.prepared = self.qk_norm is not None or self.growth is not None or self.buckets is not None \
+            or self.blend is not None or self.gated
+        self.in_dim = self.qkv_dim + (self.out_dim if self.gated else 0)
         self._slopes: Optional[torch.Tensor] = None
+        self._bias_table: Optional[torch.Tensor] = None
+        self._q_gain = self._k_gain = self._blend_weight = self._freqs = None
         self.qkv_weight = self.qkv_bias = self.proj_weight = self.proj_bias = None
         self.dtype: Optional[torch.dtype] = None
         self._table = None
@@ -71,6 +97,16 @@ class PagedAttention(Mixer):
             else {"qkv": self.qkv_dim}
         out = {f"{name}.weight": ParamSpec((rows, spec.dim)) for name, rows in pieces.items()}
         out["proj.weight"] = ParamSpec((spec.dim, self.out_dim))
+        if self.gated:
+            out["gate.weight"] = ParamSpec((self.out_dim, spec.dim))
+        if self.qk_norm is not None and self.qk_norm.gain:
+            per_head = self.qk_norm.scope == "head"
+            out["q_norm.weight"] = ParamSpec((spec.head_dim if per_head else self.q_dim,), "vector", "gain")
+            out["k_norm.weight"] = ParamSpec((spec.head_dim if per_head else self.kv_dim,), "vector", "gain")
+        if self.buckets is not None:
+            out["rel"] = ParamSpec((-1 if self.buckets.buckets is None else self.buckets.buckets, spec.n_heads), "matrix", "bias")
+        if self.blend is not None:
+            out["vmix"] = ParamSpec((), "vector", "fraction")
         if spec.bias:
             out.update({f"{name}.bias": ParamSpec((rows,), "vector", "bias") for name, rows in pieces.items()})
             out["proj.bias"] = ParamSpec((spec.dim,), "vector", "bias")
@@ -78,7 +114,7 @@ class PagedAttention(Mixer):
 
     def cache_spec(self) -> CacheSpec:
         return CacheSpec(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window,
-                         self.value_dim if self.value_dim != self.spec.head_dim else None)
+                         self.value_dim if self.value_dim != self.spec.head_dim else None, getattr(self.spec, "chunk", None))
 
     def bind(self, tensors, dtype, device) -> None:
         spec = self.spec
@@ -96,6 +132,21 @@ class PagedAttention(Mixer):
         if self.spec.bias:
             self.qkv_bias = fused("bias").to(dtype=torch.float32).contiguous()
             self.proj_bias = tensors["proj.bias"].to(device=device, dtype=torch.float32).contiguous()
+        if self.gated:
+            # the gate's rows behind those of q, k and v: one launch projects all four (the gate has no bias)
+            self.qkv_weight = torch.cat([self.qkv_weight, tensors["gate.weight"].to(device)], dim=0).contiguous()
+            if self.qkv_bias is not None:
+                self.qkv_bias = torch.cat([self.qkv_bias, torch.zeros(self.out_dim, dtype=torch.float32, device=device)]).contiguous()
+        if self.qk_norm is not None and self.qk_norm.gain:
+            self._q_gain = tensors["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+            self._k_gain = tensors["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+        if self.buckets is not None:
+            # rel [buckets, H] -> the bias by distance [H, distances]: the kernels look a distance up, not its bucket
+            buckets = self.buckets.sized(tensors["rel"].shape[0])
+            index = torch.tensor([buckets.bucket(n) for n in range(buckets.distances())], dtype=torch.long, device=device)
+            self._bias_table = tensors["rel"].to(device=device, dtype=torch.float32)[index].t().contiguous()
+        if self.blend is not None:
+            self._blend_weight = tensors["vmix"].to(device=device, dtype=torch.float32).reshape(1).contiguous()
         if self.distance is not None:
             self._slopes = torch.tensor(self.distance.values(spec.n_heads), dtype=torch.float32, device=device)
         if int(getattr(self.position, "axes", 1)) != 1:
@@ -105,7 +156,18 @@ class PagedAttention(Mixer):
         if rotation is None and callable(getattr(self.position, "table", None)) and self.position.table(device) is not None:
             raise ValueError(f"the position encoding {getattr(spec.position, 'kind', '?')!r} holds a table but offers no "
                              f"rotation(): attention would not know which channels to pair")
-        if rotation is not None:
+        if rotation is not None and getattr(rotation, "frequencies", None) is not None:
+            freqs = rotation.frequencies
+            if rotation.pairing not in core.ROTARY_PAIRINGS:
+                raise ValueError(f"attention cannot apply a rotation with pairing {rotation.pairing!r}; known: "
+                                 f"{', '.join(sorted(core.ROTARY_PAIRINGS))}")
+            if freqs.dtype != torch.float32 or freqs.dim() != 1 or 2 * freqs.numel() > spec.head_dim:
+                raise ValueError(f"a rotation's frequencies must be fp32 [R / 2] with R at most the head size {spec.head_dim}")
+            if self.unit_norm_eps is not None or self.sink is not None or self.distance is not None:
+                raise ValueError("attention with unit-norm queries and keys, distance slopes or a sink takes no rotation")
+            self._freqs, self._pairing, self._table = freqs.to(device).contiguous(), rotation.pairing, None
+            self.prepared = True
+        elif rotation is not None:
             table = rotation.table
             if rotation.pairing not in core.ROTARY_PAIRINGS:
                 raise ValueError(f"attention cannot apply a rotation with pairing {rotation.pairing!r}; known: "
@@ -113,9 +175,9 @@ class PagedAttention(Mixer):
             if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] % 2 or table.shape[1] > self.spec.head_dim:
                 raise ValueError(f"a rotation's table must be fp32 [positions, R] with R even and at most the head size "
                                  f"{self.spec.head_dim}, got {tuple(table.shape)} {table.dtype}")
-            if self.extended:
-                raise ValueError("attention with values of another size, unit-norm queries and keys, distance slopes or a "
-                                 "sink takes no rotation")
+            if self.extended or self.prepared:
+                raise ValueError("attention with values of another size, normalised queries and keys, a distance bias, a sink, "
+                                 "blended values or an output gate takes no rotation from a table (one from frequencies it does)")
             self._table, self._pairing = table.to(device).contiguous(), rotation.pairing
         else:
             self._table, self._pairing = None, "halves"
@@ -131,7 +193,7 @@ class PagedAttention(Mixer):
     # The three stages are also offered one by one, so that a block may fuse the first with its
     # norm and the last with its feed-forward (see ``Mixer.input_projection``).
     def input_projection(self):
-        return self.qkv_weight, self.qkv_bias, self.qkv_dim
+        return self.qkv_weight, self.qkv_bias, self.in_dim
 
     def output_projection(self):
         return self.proj_weight, self.proj_bias
@@ -140,6 +202,7 @@ class PagedAttention(Mixer):
         """One token per row in bf16 with a rotation by halves: the decode kernel then rotates q and
         k and stores k and v itself."""
         return self.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None and not self.extended \
+            and not self.prepared \
             and self._pairing == "halves"          # the MFMA-path kernels turn halves; the generic one any pairing
 
     def takes_beside(self, job, batch, cache: LayerCache) -> bool:
@@ -155,6 +218,10 @@ class PagedAttention(Mixer):
         n = qkv.shape[0]
         group = batch.groups[cache.group]
         out = batch.workspace.get("attn.out", (n, self.out_dim), self.dtype)
+        if self.prepared:
+            if beside is not None:
+                self._alone(beside)
+            return self._attend_prepared(qkv, batch, cache, group, out)
         if self.extended:
             if beside is not None:
                 self._alone(beside)
@@ -209,16 +276,56 @@ class PagedAttention(Mixer):
                                self._slopes, self.sink)
         return out
 
+    def _attend_prepared(self, projected, batch, cache: LayerCache, group, out):
+        """Queries, keys and values made ready by one kernel (norms, rotation, factor, blend, cache write), attention with
+        the distance table where there is one, then the output gate. ``projected``: ``[n, q | k | v (| gate)]``."""
+        spec = self.spec
+        n = projected.shape[0]
+        qkv = projected[:, :self.qkv_dim] if self.gated else projected
+        slots = group.slots if cache.writes else None
+        other = None
+        if self.blend is not None:
+            # the source layer's values of this step's tokens: scratch of the step, at a fixed address under graphs
+            other = batch.workspace.get("shared." + self.blend.name, (n, self.v_dim), self.dtype)
+        norm = self.qk_norm
+        core.qkv_prepare(qkv, batch.positions, slots, cache.k, cache.v, spec.n_heads, spec.n_kv_heads, spec.head_dim,
+                         self.value_dim, group.page_size, norm.scope if norm is not None else None, self._q_gain, self._k_gain,
+                         float(norm.eps) if norm is not None else 0.0, self._freqs, self._pairing,
+                         (self.growth.coef, self.growth.every) if self.growth is not None else None,
+                         self.blend.role if self.blend is not None else None, other, self._blend_weight)
+        done = False
+        if qkv.dtype == torch.bfloat16:
+            from ..ops import fast
+            if self.extended:
+                done = fast.attention_biased_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo,
+                                                  batch.kv_hi, out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim,
+                                                  self.value_dim, batch.positions, None, None, batch, bias_table=self._bias_table)
+            else:
+                paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
+                                self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
+                done = True
+        if not done:
+            core.attention_generic(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
+                                   self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, self.value_dim, batch.positions,
+                                   None, None, bias_table=self._bias_table)
+        if self.gated:
+            core.gate_mul(out, projected[:, self.qkv_dim:])
+        return out
+
     @staticmethod
     def _alone(job) -> None:
         """A job that was promised a place in the attention launch and did not get one after all."""
         linear(job.a, job.weight, job.bias, job.out, act=job.act)
 
-    def forward(self, h, batch, cache: LayerCache, residual) -> None:
-        qkv = batch.workspace.get("attn.qkv", (h.shape[0], self.qkv_dim), self.dtype)
+    def mix(self, h, batch, cache: LayerCache, out, accumulate: bool) -> None:
+        """The mixer's output written into (or added to) fp32 ``out``."""
+        qkv = batch.workspace.get("attn.qkv", (h.shape[0], self.in_dim), self.dtype)
         linear(h, self.qkv_weight, self.qkv_bias, qkv)
-        out = self.attend(qkv, batch, cache)
-        linear(out, self.proj_weight, self.proj_bias, residual, accumulate=True)
+        mixed = self.attend(qkv, batch, cache)
+        linear(mixed, self.proj_weight, self.proj_bias, out, accumulate=accumulate)
+
+    def forward(self, h, batch, cache: LayerCache, residual) -> None:
+        self.mix(h, batch, cache, residual, True)
 
 
 register_mixer("attention", PagedAttention)

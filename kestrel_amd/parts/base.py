@@ -63,10 +63,13 @@ class Rotation:
     ``p``, then their sines; the first ``R`` channels of every query and key head are turned.
     ``pairing``: which two channels angle ``i`` turns: ``"halves"`` = ``i`` and ``i + R / 2``,
     ``"interleaved"`` = ``2 i`` and ``2 i + 1``.
+    ``frequencies``: instead of a table, fp32 ``[R / 2]``: angle ``i`` of position ``p`` is ``p * frequencies[i]``, computed
+    by the kernel (``table`` is then ``None``).
     """
 
-    table: torch.Tensor
+    table: Optional[torch.Tensor]
     pairing: str = "halves"
+    frequencies: Optional[torch.Tensor] = None
 
 
 class PositionEncoding(Part):

@@ -21,7 +21,7 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
     from ..ops.linear import linear
 
     n = x.shape[0]
-    if block.dtype != torch.bfloat16 or n > fast.SKINNY_MAX_ROWS:
+    if block.dtype != torch.bfloat16 or n > fast.SKINNY_MAX_ROWS or block.feed_forward is None:
         return False
     m_in, f_in = block.mixer.input_projection(), block.feed_forward.input_projection()
     m_out, f_out = block.mixer.output_projection(), block.feed_forward.output_projection()
@@ -75,7 +75,8 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
 
 
 def _parallel(block: "Block", x, batch, cache, normed=None, then=None):
-    """``x + mixer(norm(x)) + ff(norm(x))``: both branches read the same normalised input.
+    """``x + mixer(norm(x)) + ff(norm(x))``: both branches read the same normalised input (a block without a
+    feed-forward has the first branch only).
 
     Reference: ``kestrel/models/moondream/text.py:222-275``.
     """
@@ -87,7 +88,8 @@ def _parallel(block: "Block", x, batch, cache, normed=None, then=None):
         h = batch.workspace.get("block.h", tuple(x.shape), block.dtype)
         block.norm.forward(x, h)
     block.mixer.forward(h, batch, cache, x)
-    block.feed_forward.forward(h, batch, x)
+    if block.feed_forward is not None:
+        block.feed_forward.forward(h, batch, x)
     return None
 
 
@@ -223,7 +225,7 @@ class Block:
         if spec.arrangement == "sequential" and self.norm2 is None:
             raise ValueError("the sequential arrangement needs norm2")
         self.mixer = build_part("mixer", spec.mixer)
-        if spec.feed_forward is None and spec.arrangement != "parallel_two_norms":
+        if spec.feed_forward is None and spec.arrangement not in ("parallel_two_norms", "parallel"):
             raise ValueError(f"the {spec.arrangement} arrangement needs a feed-forward")
         if spec.arrangement == "parallel_two_norms" and spec.feed_forward is not None and self.norm2 is None:
             raise ValueError("the parallel_two_norms arrangement needs norm2 for its feed-forward")

@@ -1,4 +1,4 @@
-"""Dense feed-forward: two linears around an activation."""
+"""Dense feed-forwards: two linears around an activation, plain or gated."""
 
 from __future__ import annotations
 
@@ -6,9 +6,9 @@ from typing import Dict, Optional
 
 import torch
 
-from ..ops.linear import activation_code, linear
+from ..ops.linear import ACT_GATED, activation_code, linear, linear_gated, pair_rows
 from .base import FeedForward, register_feed_forward
-from .specs import DenseFeedForwardSpec, ParamSpec
+from .specs import DenseFeedForwardSpec, GatedFeedForwardSpec, ParamSpec
 
 
 class DenseFeedForward(FeedForward):
@@ -54,4 +54,47 @@ class DenseFeedForward(FeedForward):
         linear(hidden, self.fc2_weight, self.fc2_bias, residual, accumulate=True)
 
 
+class GatedFeedForward(FeedForward):
+    """``down(act(gate h) * (up h))``: the rows of ``gate`` and ``up`` are laid in pairs when the weights are bound, so
+    that one linear computes both and takes the product in its epilogue (``ops.linear.linear_gated``)."""
+
+    replays_every_step = True
+
+    def __init__(self, spec: GatedFeedForwardSpec) -> None:
+        super().__init__(spec)
+        self.act = activation_code(spec.activation)
+        self.pairs = self.pair_bias = self.down_weight = self.down_bias = None
+        self.dtype: Optional[torch.dtype] = None
+
+    def params(self) -> Dict[str, ParamSpec]:
+        spec = self.spec
+        out = {"gate.weight": ParamSpec((spec.hidden_dim, spec.dim)), "up.weight": ParamSpec((spec.hidden_dim, spec.dim)),
+               "down.weight": ParamSpec((spec.dim, spec.hidden_dim))}
+        if spec.bias:
+            out.update({"gate.bias": ParamSpec((spec.hidden_dim,), "vector", "bias"), "up.bias": ParamSpec((spec.hidden_dim,), "vector", "bias"),
+                        "down.bias": ParamSpec((spec.dim,), "vector", "bias")})
+        return out
+
+    def bind(self, tensors, dtype, device) -> None:
+        self.dtype = dtype
+        self.pairs = pair_rows(tensors["gate.weight"].to(device), tensors["up.weight"].to(device))
+        self.down_weight = tensors["down.weight"].to(device).contiguous()
+        if self.spec.bias:
+            self.pair_bias = pair_rows(tensors["gate.bias"].to(device=device, dtype=torch.float32),
+                                       tensors["up.bias"].to(device=device, dtype=torch.float32))
+            self.down_bias = tensors["down.bias"].to(device=device, dtype=torch.float32).contiguous()
+
+    def input_projection(self):
+        return self.pairs, self.pair_bias, self.spec.hidden_dim, self.act | ACT_GATED
+
+    def output_projection(self):
+        return self.down_weight, self.down_bias
+
+    def forward(self, h, batch, residual) -> None:
+        hidden = batch.workspace.get("ff.hidden", (h.shape[0], self.spec.hidden_dim), self.dtype)
+        linear_gated(h, self.pairs, self.pair_bias, hidden, self.act)
+        linear(hidden, self.down_weight, self.down_bias, residual, accumulate=True)
+
+
 register_feed_forward("dense", DenseFeedForward)
+register_feed_forward("gated_dense", GatedFeedForward)

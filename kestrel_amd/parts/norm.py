@@ -1,4 +1,4 @@
-"""LayerNorm with gain and optional shift; statistics in fp32."""
+"""LayerNorm with gain and optional shift, and the root-mean-square norm with gain; statistics in fp32."""
 
 from __future__ import annotations
 
@@ -43,4 +43,26 @@ class LayerNorm(Norm):
         return self.weight, self.bias, float(self.spec.eps)
 
 
+class RMSNorm(Norm):
+    """``x / sqrt(mean(x^2) + eps) * weight`` over the last axis: no mean is taken off, no shift is added, the
+    weight is used as stored (not as one plus it). It offers no ``layernorm_operands``, so it always runs in a
+    launch of its own."""
+
+    replays_every_step = True
+
+    def __init__(self, spec: NormSpec) -> None:
+        super().__init__(spec)
+        self.weight: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.spec.dim,), "vector", "gain")}
+
+    def bind(self, tensors, dtype, device) -> None:
+        self.weight = tensors["weight"].to(device=device, dtype=torch.float32).contiguous()
+
+    def forward(self, x, out, rows=None) -> None:
+        core.rmsnorm(x, self.weight, self.spec.eps, out, rows)
+
+
 register_norm("layernorm", LayerNorm)
+register_norm("rmsnorm", RMSNorm)

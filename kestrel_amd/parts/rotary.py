@@ -44,6 +44,46 @@ class NeoxRotary(PositionEncoding):
         return self._table
 
 
+def rotary_frequencies(rotary_dim: int, theta: float, scaling=None):
+    """``f_i = theta ** (-2 i / rotary_dim)`` for the ``rotary_dim / 2`` pairs, rescaled by wavelength where a
+    ``WavelengthScaling`` is given (long wavelengths divided by its factor, short ones kept, a linear blend between)."""
+    import math
+
+    out = []
+    for i in range(rotary_dim // 2):
+        f = float(theta) ** (-2.0 * i / rotary_dim)
+        if scaling is not None:
+            wavelength = 2.0 * math.pi / f
+            if wavelength > scaling.original / scaling.low:
+                f = f / scaling.factor
+            elif wavelength >= scaling.original / scaling.high:
+                s = (scaling.original / wavelength - scaling.low) / (scaling.high - scaling.low)
+                f = (1.0 - s) * f / scaling.factor + s * f
+        out.append(f)
+    return out
+
+
+class FrequencyRotary(PositionEncoding):
+    """A rotation given by its frequencies alone: the kernels compute the angle ``place * f_i`` and its cosine and sine
+    in fp32 themselves, so there is no table and no longest sequence. ``spec.pairing`` says which channels angle ``i``
+    turns (``"halves"`` or ``"interleaved"``), ``spec.scaling`` rescales the frequencies by wavelength."""
+
+    replays_every_step = True
+
+    def __init__(self, spec: PositionSpec) -> None:
+        super().__init__(spec)
+        if spec.rotary_dim <= 0 or spec.rotary_dim % 2:
+            raise ValueError(f"rotary_dim {spec.rotary_dim} must be even and positive")
+        self._freqs: Optional[torch.Tensor] = None
+
+    def rotation(self, device: torch.device) -> Optional[Rotation]:
+        spec = self.spec
+        if self._freqs is None or self._freqs.device != device:
+            values = rotary_frequencies(spec.rotary_dim, spec.theta, getattr(spec, "scaling", None))
+            self._freqs = torch.tensor(values, dtype=torch.float64).to(torch.float32).to(device)
+        return Rotation(None, getattr(spec, "pairing", "halves"), self._freqs)
+
+
 class NoPosition(PositionEncoding):
     """Encodes nothing (a mixer whose order comes from elsewhere)."""
 
@@ -51,4 +91,5 @@ class NoPosition(PositionEncoding):
 
 
 register_position("rotary_neox", NeoxRotary)
+register_position("rotary", FrequencyRotary)
 register_position("none", NoPosition)

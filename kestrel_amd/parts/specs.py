@@ -20,8 +20,9 @@ class ParamSpec:
 
     ``role`` fixes how the tensor is held and initialised: ``matrix`` (2-D weight,
     model precision), ``vector`` (bias or gain), ``table`` (integer table, int32).
-    ``init`` names the random-weights recipe: ``normal``, ``bias``, ``gain`` (around 1)
-    or ``shift`` (around 0).
+    ``init`` names the random-weights recipe: ``normal``, ``bias``, ``gain`` (around 1),
+    ``shift`` (around 0) or ``fraction`` (around one half, inside 0 .. 1). An extent of -1 in ``shape`` leaves that
+    size to the weights file (the part then reads it off the tensor it is bound to).
     """
 
     shape: Tuple[int, ...]
@@ -38,13 +39,28 @@ class NormSpec:
 
 
 @dataclass(frozen=True)
+class WavelengthScaling:
+    """Rotary frequencies rescaled by wavelength ``l = 2 pi / f``: kept where ``l < original / high``, divided by
+    ``factor`` where ``l > original / low``, and in between ``(1 - s) f / factor + s f`` with
+    ``s = (original / l - low) / (high - low)``."""
+
+    factor: float
+    low: float
+    high: float
+    original: float
+
+
+@dataclass(frozen=True)
 class PositionSpec:
-    """Position encoding applied inside a mixer. ``kind`` ``none`` encodes nothing."""
+    """Position encoding applied inside a mixer. ``kind`` ``none`` encodes nothing. ``pairing`` and ``scaling`` are
+    read by the kind ``rotary`` (angles computed from frequencies, no table and so no longest sequence)."""
 
     kind: str
     rotary_dim: int = 0
     theta: float = 0.0
     max_positions: int = 0
+    pairing: str = "halves"
+    scaling: Optional[WavelengthScaling] = None
 
 
 @dataclass(frozen=True)
@@ -78,11 +94,78 @@ class DistanceSlopes:
 
 
 @dataclass(frozen=True)
+class QKNorm:
+    """Queries and keys divided by a root mean square ``sqrt(mean(square) + eps)`` before rotation and scores: over
+    every head by itself (``scope`` ``"head"``, gains of one head's size shared by all heads) or over the whole
+    projection of a token (``"projection"``, gains of the projection's size). ``gain`` ``False``: no gains."""
+
+    scope: str
+    eps: float
+    gain: bool = True
+
+
+@dataclass(frozen=True)
+class QueryGrowth:
+    """Queries at place ``p`` multiplied by ``1 + coef * ln(floor((p + 1) / every) + 1)``."""
+
+    coef: float
+    every: int
+
+
+@dataclass(frozen=True)
+class DistanceBuckets:
+    """A learned bias on attention scores by distance and head, ``rel[bucket(i - j), h]`` with ``rel`` ``[buckets, H]``:
+    with ``half = buckets // 2``, ``bucket(n) = n`` for ``n < half``, else
+    ``min(buckets - 1, half + floor(ln(n / half) / ln(far / half) * (buckets - half)))``. ``buckets`` ``None``: the
+    number of rows of ``rel`` as stored says (``sized(rows)`` then gives the specification with the number in it)."""
+
+    buckets: Optional[int]
+    far: float
+
+    def sized(self, buckets: int) -> "DistanceBuckets":
+        return DistanceBuckets(int(buckets), self.far)
+
+    def bucket(self, n: int) -> int:
+        import math
+
+        half = self.buckets // 2
+        if n < half:
+            return n
+        return min(self.buckets - 1, half + int(math.floor(math.log(n / half) / math.log(self.far / half) * (self.buckets - half))))
+
+    def distances(self) -> int:
+        """Distances ``0 .. distances() - 1`` have buckets of their own to be looked up; every larger one falls into
+        the last bucket, like ``distances() - 1`` does."""
+        import math
+
+        half = self.buckets // 2
+        if self.buckets < 2 or not self.far > half:
+            raise ValueError(f"distance buckets: {self.buckets} buckets need a far distance above {half}, got {self.far}")
+        n = int(math.ceil(self.far))
+        while n > 0 and self.bucket(n - 1) == self.buckets - 1:
+            n -= 1
+        return n + 1
+
+
+@dataclass(frozen=True)
+class ValueBlend:
+    """Values of a layer blended with those another layer computed for the same token: the layer with ``role``
+    ``"source"`` leaves its values for the step under ``name``; a layer with ``role`` ``"blend"`` replaces its own by
+    ``(1 - w) v + w v_source`` with its learned scalar ``w`` before they are cached. (A source holds the scalar too
+    and does not use it.)"""
+
+    role: str
+    name: str = "values"
+
+
+@dataclass(frozen=True)
 class CacheSpec:
     """What an attention mixer keeps per token: keys and values of ``n_kv_heads`` x ``head_dim``.
 
     ``window`` = number of most recent positions a query reads (``None``: all), which
-    lets the cache manager give back pages that have fallen out of it.
+    lets the cache manager give back pages that have fallen out of it. ``chunk`` = size of the chunks, counted
+    from position 0, outside of which a query reads nothing (``None``: none): pages before the chunk of the next
+    position go back as well.
 
     The cache manager asks a specification three things and nothing else, so a mixer that keeps
     something other than keys and values per token (one latent, another layout) brings a
@@ -96,6 +179,21 @@ class CacheSpec:
     head_dim: int
     window: Optional[int] = None
     value_dim: Optional[int] = None     # size of a value head where it is not the keys' (``None``: ``head_dim``)
+    chunk: Optional[int] = None
+
+    def first_visible(self, position: int) -> int:
+        """The lowest key position that a query at ``position`` reads."""
+        lo = 0
+        if self.window is not None:
+            lo = max(lo, position + 1 - self.window)
+        if self.chunk is not None:
+            lo = max(lo, position // self.chunk * self.chunk)
+        return lo
+
+    @property
+    def bounded(self) -> bool:
+        """Whether queries stop reading old keys at some point (pages can then be given back)."""
+        return self.window is not None or self.chunk is not None
 
     def page_tensors(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
         # values are kept transposed inside a page: eight consecutive keys of one channel are 16
@@ -106,7 +204,8 @@ class CacheSpec:
     @property
     def group_key(self) -> Tuple:
         value_dim = self.head_dim if self.value_dim is None else self.value_dim
-        return ("kv", self.n_kv_heads, self.head_dim, self.window) + ((value_dim,) if value_dim != self.head_dim else ())
+        return ("kv", self.n_kv_heads, self.head_dim, self.window) + ((value_dim,) if value_dim != self.head_dim else ()) \
+            + ((("chunk", self.chunk),) if self.chunk is not None else ())
 
 
 @dataclass(frozen=True)
@@ -139,6 +238,18 @@ class AttentionSpec:
     distance_slopes: Optional[DistanceSlopes] = None
     # one more term ``exp(sink)`` in the softmax's denominator that carries no value (``None``: none)
     sink: Optional[float] = None
+    # a query reads only keys of its own chunk of this many positions (chunks counted from position 0)
+    chunk: Optional[int] = None
+    # queries and keys normalised, with learned gains, over a head or over the whole projection
+    qk_norm: Optional[QKNorm] = None
+    # a factor on the queries that grows with the place
+    query_growth: Optional[QueryGrowth] = None
+    # a learned bias per bucket of distance and head (tensor ``rel``)
+    distance_buckets: Optional[DistanceBuckets] = None
+    # values blended with those of another layer of the step (tensor ``vmix``)
+    value_blend: Optional[ValueBlend] = None
+    # the concatenated heads multiplied by ``sigmoid(gate.weight @ input)`` before the output projection
+    output_gate: bool = False
 
 
 @dataclass(frozen=True)
@@ -151,10 +262,48 @@ class DenseFeedForwardSpec:
 
 
 @dataclass(frozen=True)
+class GatedFeedForwardSpec:
+    """``down(act(gate h) * (up h))``."""
+
+    kind: str
+    dim: int
+    hidden_dim: int
+    activation: str = "gelu_tanh"
+    bias: bool = False
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """A recurrent mixer whose state per head is a matrix ``[head_dim, value_dim]`` with a normaliser and a running
+    maximum, written through exponential input and forget gates (``parts/matrix_memory.py``)."""
+
+    kind: str
+    dim: int
+    n_heads: int
+    head_dim: int
+    value_dim: int
+    gate_cap: float                 # gate pre-activations pass through ``cap * tanh(x / cap)``
+    eps: float                      # of the norm of every head's read-out
+    output_gate: bool = True
+
+
+@dataclass(frozen=True)
+class BranchesSpec:
+    """Mixers side by side on the same input: the result is ``sum_i weights[i] * rms(branch_i(h)) * gain_i``, every
+    branch's output normalised over the model width (``eps``) with a gain of its own."""
+
+    kind: str
+    dim: int
+    branches: Tuple[object, ...]
+    weights: Tuple[float, ...]
+    eps: float
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One block: its parts, how they are arranged, and where their tensors are named.
 
-    ``arrangement``: ``parallel`` = ``x + mixer(norm(x)) + ff(norm(x))`` (one norm);
+    ``arrangement``: ``parallel`` = ``x + mixer(norm(x)) + ff(norm(x))`` (one norm; ``feed_forward`` may be ``None``);
     ``sequential`` = ``x += mixer(norm(x)); x += ff(norm2(x))``;
     ``parallel_two_norms`` = ``x + residual_scale * (mixer(norm(x)) + ff(norm2(x)))``, both norms of the same ``x``
     (``feed_forward`` and ``norm2`` may be ``None`` there: a layer of a mixer alone).

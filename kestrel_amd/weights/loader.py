@@ -148,7 +148,8 @@ def load_tensors(path, expected: Dict[str, ParamSpec], run_dtype: torch.dtype, d
                 missing.append(name)
                 continue
             shape = handle.shape(key)
-            if shape != tuple(spec.shape):
+            # (an extent of -1 in the specification: the file decides, and the part reads the size off the tensor)
+            if len(shape) != len(spec.shape) or any(want not in (-1, have) for have, want in zip(shape, spec.shape)):
                 mismatched.append(f"{name}: stored {list(shape)}, the model needs {list(spec.shape)}")
         if missing or unexpected or mismatched:
             raise WeightsError(path, sorted(missing), sorted(unexpected), mismatched)

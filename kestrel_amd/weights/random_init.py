@@ -44,6 +44,9 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, recipe: InitRecipe, dev
     gen.manual_seed(_seed_of(seed, name))
     if spec.role == "table":
         raise ValueError(f"{name}: no random recipe for integer tables")
+    if any(extent < 0 for extent in spec.shape):
+        raise ValueError(f"{name}: the configuration leaves an extent of this tensor to the weights file {tuple(spec.shape)}; "
+                         f"name it in the configuration to write random weights")
     noise = torch.randn(tuple(spec.shape), generator=gen, dtype=torch.float32, device=device)
     if spec.init == "normal":
         return noise * recipe.std
@@ -53,6 +56,8 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, recipe: InitRecipe, dev
         return 1.0 + noise * recipe.gain_std
     if spec.init == "shift":
         return noise * recipe.shift_std
+    if spec.init == "fraction":
+        return (0.5 + 0.15 * noise).clamp(0.05, 0.95)
     raise ValueError(f"{name}: unknown init {spec.init!r}")
 
 
