@@ -213,10 +213,10 @@ class ModelRunner:
                  max_graph_batch: Optional[int] = None, max_positions: Optional[int] = None) -> None:
         self.model, self.cache, self.device = model, cache, device
         # the longest sequence a request may grow to: what the model allows (a design without a bound of its own names
-        # a very large number) and what the caller allows; a row can never hold more than the pool does, which bounds
-        # the width of block tables and the longest row that graphs are captured for
+        # a large number) and what the caller allows; it fixes the width of the block tables of captured steps (a row
+        # whose window has passed keeps its logical pages in the table, so the pool's size is no bound)
         self.max_positions = min(int(model.plan.max_positions), int(max_positions or model.plan.max_positions))
-        self._longest_row = min(self.max_positions, cache.n_pages * cache.page_size)
+        self._longest_row = self.max_positions
         self.max_tokens_per_step = max_tokens_per_step
         self.workspace = Workspace(device)
         self.layer_caches = cache.layer_caches()

@@ -40,9 +40,10 @@ NAME = "bogivik"
 MLP_ACTIVATION = "gelu_tanh"
 BRANCH_WEIGHTS = (0.5, 0.5)            # the parallel mixer is half the sum of its two normalised branches
 VALUE_BLEND_NAME = "first_values"
-# The design has no longest sequence of its own (no table depends on one): a request may grow as far as the
-# engine's cache lets it. ``config.json`` may name a bound (``max_positions``); without one this stands.
-DEFAULT_MAX_POSITIONS = 1 << 20
+# The design has no longest sequence of its own (no table depends on one). ``config.json`` may name a bound
+# (``max_positions``); without one this stands, and the engine's ``max_seq_len`` narrows it (captured steps carry
+# block tables of that many positions).
+DEFAULT_MAX_POSITIONS = 1 << 17
 
 
 def _positive_int(where: str, value) -> int:
