@@ -18,6 +18,8 @@ greedy requests of such a run are compared, token by token, with the plain imple
 ``--workload compare-vimesun`` measures the Vimesun design beside the Moondream decoder at equal sizes (width,
 feed-forward, heads, head size, runs of layers, vocabulary; random weights): a prompt alone and decode steps at batch 1,
 8 and 64 through the same step function, each with its share of the roofline (``--compare-sizes``, ``--compare-model``).
+``--workload compare-bogivik`` does the same for the Bogivik design (layers of attention with a distance bias and a
+layer of chunked attention beside a matrix memory) at sizes of its own (``BOGIVIK_SIZES``).
 """
 
 from __future__ import annotations
@@ -185,6 +187,139 @@ def run_compare(args, dtype, device) -> dict:
             "ms_per_step": lead["decode_b8"]["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": args.dtype, "data": "synthetic (seeded random token ids, random weights N(0,0.02))",
             "config": {"model": "vimesun and moondream2-text at equal sizes", "sizes": {k: COMPARE_SIZES[k] for k in out},
+                       "global_batch": 8, "seq_len": context, "vocab_size": COMPARE_VOCAB, "parallelism": "single-gpu"},
+            "compare": out}
+
+
+# Sizes at which Bogivik is measured beside the Moondream decoder: width, gated feed-forward (Moondream's plain one gets
+# one and a half times the hidden size: the same weights), heads, kv heads, head size (keys and values), the chunk of the
+# chunked branch, heads and head sizes of the matrix memory, and the order of layers (a: attention, p: parallel).
+BOGIVIK_SIZES = {
+    "w2048": dict(width=2048, ff=5632, heads=32, kv_heads=8, head=64, chunk=1024, memory=(8, 64, 256), order="aapa"),
+    "w4096": dict(width=4096, ff=7168, heads=32, kv_heads=8, head=128, chunk=2048, memory=(16, 64, 256), order="apa"),
+}
+
+
+def bogivik_models(size: dict, positions: int):
+    """``{name: (config dict, registry name)}`` of Bogivik and of the Moondream decoder at one size."""
+    h, g, d, w = size["heads"], size["kv_heads"], size["head"], size["width"]
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    attention = {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "bias_max": 128, "buckets": 32,
+                 "q_temp": {"coef": 0.5, "every": 64}, "v_mix": True}
+    mh, md, mdv = size["memory"]
+    parallel = {"left": {"heads": h, "kv_heads": g, "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": size["chunk"]},
+                         "rot": {"base": 10000.0, "dims": d, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+                "right": {"heads": mh, "dim": md, "vdim": mdv, "gate_cap": 15.0}}
+    layers = [{"type": "attention", "mixer": dict(attention), "mlp": mlp} if kind == "a" else
+              {"type": "parallel", "mixer": parallel, "mlp": mlp} for kind in size["order"]]
+    bogivik = {"architecture": "Bogivik", "vocab": COMPARE_VOCAB, "width": w, "norm": {"eps": 1e-6}, "max_positions": positions,
+               "layers": layers}
+    moondream = {"text": {"dim": w, "ff_dim": size["ff"] * 3 // 2, "n_layers": len(size["order"]), "vocab_size": COMPARE_VOCAB,
+                          "max_context": positions, "n_heads": h, "n_kv_heads": g, "head_dim": d, "rotary_dim": d // 2,
+                          "rope_theta": 10000.0, "prefix_attn": 0, "layer_norm_eps": 1e-5}}
+    return {"bogivik": (bogivik, "bogivik"), "moondream2": (moondream, "moondream2")}
+
+
+def design_facts(net):
+    """What the roofline of any model of the package needs, read off its plan: the weights of its linears (every matrix
+    but the embedding table), and per layer the sizes of its attention (heads, kv heads, key and value size, window,
+    chunk) and of its matrix memory (heads, key and value size)."""
+    from types import SimpleNamespace
+
+    plan = net.plan
+    embedding = plan.names["embedding"]
+    linear = sum(int(__import__("math").prod(p.shape)) for name, p in net.params().items() if p.role == "matrix" and name != embedding)
+    attention, memory = [], []
+
+    def walk(spec):
+        kind = getattr(spec, "kind", None)
+        if kind == "attention":
+            dv = spec.head_dim if getattr(spec, "value_dim", None) is None else spec.value_dim
+            attention.append((spec.n_heads, spec.n_kv_heads, spec.head_dim, dv, getattr(spec, "window", None), getattr(spec, "chunk", None)))
+        elif kind == "matrix_memory":
+            memory.append((spec.n_heads, spec.head_dim, spec.value_dim))
+        elif kind == "branches":
+            for branch in spec.branches:
+                walk(branch)
+
+    for entry in plan.schedule:
+        walk(plan.layers[entry.layer].mixer)
+    return SimpleNamespace(linear=linear, attention=attention, memory=memory, width=plan.dim, vocab=plan.vocab_size)
+
+
+def _keys_seen(place: int, window, chunk) -> int:
+    lo = 0
+    if window is not None:
+        lo = max(lo, place + 1 - window)
+    if chunk is not None:
+        lo = max(lo, place // chunk * chunk)
+    return place + 1 - lo
+
+
+def design_flops(f, tokens: int) -> float:
+    """Multiply-adds x 2 of a prompt of ``tokens`` places: the linears (the head at the last place only), score and value
+    products over the keys each place sees, the matrix memory's update and read-out (two multiply-adds a number of state)."""
+    total = 2.0 * tokens * (f.linear - f.width * f.vocab) + 2.0 * f.width * f.vocab
+    for h, _g, d, dv, window, chunk in f.attention:
+        total += 2.0 * h * (d + dv) * sum(_keys_seen(p, window, chunk) for p in range(tokens))
+    for h, d, dv in f.memory:
+        total += 2.0 * 2.0 * h * d * dv * tokens
+    return total
+
+
+def design_decode_bytes(f, batch: int, context: int, size: int) -> float:
+    """Bytes a decode step must move: every weight once, of every row the keys and values it sees, and its matrix
+    memories' fp32 state read and written."""
+    total = float(size) * f.linear
+    for _h, g, d, dv, window, chunk in f.attention:
+        total += size * batch * g * (d + dv) * _keys_seen(context, window, chunk)
+    for h, d, dv in f.memory:
+        total += 2.0 * 4 * batch * h * (d * dv + d + 1)
+    return total
+
+
+def run_compare_bogivik(args, dtype, device) -> dict:
+    """Bogivik beside the Moondream decoder at equal sizes, through the same step function."""
+    from types import SimpleNamespace
+
+    import torch
+
+    size_bytes = 2 if dtype == torch.bfloat16 else 4
+    context, tokens = args.context, args.prefill_tokens
+    positions = max(context + args.steps + args.warmup + 16, tokens)
+    labels = [label for label in args.compare_sizes.split(",") if label in BOGIVIK_SIZES] or list(BOGIVIK_SIZES)
+    out = {}
+    for label in labels:
+        out[label] = {}
+        for name, (config, registry_name) in bogivik_models(BOGIVIK_SIZES[label], positions).items():
+            if args.compare_model not in ("both", name):
+                continue
+            net, _typed = build_from_config(config, registry_name, dtype, device)
+            f = design_facts(net)
+            shim = SimpleNamespace(prefix_attn=0, dim=f.width, vocab_size=f.vocab, n_kv_heads=1, head_dim=1, n_layers=1)
+            entry = {}
+            if not args.skip_prefill:
+                seconds, best = time_prefill(net, shim, tokens, repeats=5)
+                flops = design_flops(f, tokens)
+                entry["prefill"] = {"tokens": tokens, "ms": round(seconds * 1e3, 3), "best_ms": round(best * 1e3, 3),
+                                    "tok_s": round(tokens / seconds, 1), "frac_of_peak_flops": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+            for batch in [int(b) for b in args.compare_batches.split(",") if b]:
+                steps = args.steps if batch < 64 else max(16, args.steps // 4)
+                elapsed, _kv = time_decode(net, shim, batch, context, steps, min(args.warmup, 4))
+                moved = design_decode_bytes(f, batch, context, size_bytes)
+                entry[f"decode_b{batch}"] = {"ms_per_step": round(elapsed / steps * 1e3, 4), "tok_s": round(batch * steps / elapsed, 1),
+                                             "frac_of_peak_hbm": round(moved / (elapsed / steps) / PEAK_HBM, 4)}
+            out[label][name] = entry
+            del net
+            torch.cuda.empty_cache()
+    first = out[labels[0]]
+    lead = first.get("bogivik") or next(iter(first.values()))
+    key = "decode_b8" if "decode_b8" in lead else next((k for k in lead if k.startswith("decode")), None)
+    return {"metric": f"Bogivik beside the Moondream decoder at equal sizes: decode tok/s at batch 8, context {context} ({labels[0]})",
+            "value": lead[key]["tok_s"] if key else None, "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": lead[key]["ms_per_step"] if key else None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": args.dtype, "data": "synthetic (seeded random token ids, random weights N(0,0.02))",
+            "config": {"model": "bogivik and moondream2-text at equal sizes", "sizes": {k: BOGIVIK_SIZES[k] for k in out},
                        "global_batch": 8, "seq_len": context, "vocab_size": COMPARE_VOCAB, "parallelism": "single-gpu"},
             "compare": out}
 
@@ -476,13 +611,15 @@ def main() -> int:
                         help="with --workload: RuntimeConfig.tune_linears (time the vendor library's algorithms at warm-up)")
     parser.add_argument("--check", type=int, default=0,
                         help="with --workload: compare this many greedy requests with the plain implementation (for --layers 2)")
-    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun"],
+    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun", "compare-bogivik"],
                         help="decode: the benchmark's decode step (default); waves256 and mixed48 run requests through "
-                             "InferenceEngine; compare-vimesun measures the Vimesun design beside the Moondream decoder at equal sizes")
+                             "InferenceEngine; compare-vimesun and compare-bogivik measure that design beside the Moondream decoder at equal sizes")
     parser.add_argument("--compare-sizes", default="w2048,w2048-window,w4096-gqa,w2560-v",
                         help="with --workload compare-vimesun: which of the sizes, with commas between them")
-    parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "moondream2"],
-                        help="with --workload compare-vimesun: one of the two designs only (for profiling)")
+    parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "bogivik", "moondream2"],
+                        help="with --workload compare-*: one of the two designs only (for profiling)")
+    parser.add_argument("--compare-batches", default="1,8,64", help="with --workload compare-bogivik: batch sizes of the decode steps")
+    parser.add_argument("--skip-prefill", action="store_true", help="with --workload compare-bogivik: decode steps only")
     parser.add_argument("--max-batch-size", type=int, default=None, help="for the workloads through the entry point")
     parser.add_argument("--linears", default="library", choices=["library", "own"],
                         help="linears of more than 64 rows (a prompt's): through hipBLASLt (the engine's default) or "
@@ -510,6 +647,9 @@ def main() -> int:
         args.layers = sizes["n_layers"]
     if args.workload == "compare-vimesun":
         print(json.dumps(run_compare(args, dtype, device)))
+        return 0
+    if args.workload == "compare-bogivik":
+        print(json.dumps(run_compare_bogivik(args, dtype, device)))
         return 0
     if args.workload != "decode":
         print(json.dumps(run_workload(args, dict(SIZES[args.sizes]))))

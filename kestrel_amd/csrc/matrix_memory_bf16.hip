@@ -1,0 +1,342 @@
+// The gated matrix memory over prompt portions on the matrix cores (bf16 operands, fp32 sums, fp32 state).
+//
+// The recurrence of a head (state S [d, dv], normaliser n [d], running maximum m; see mixer_parts.hip),
+//     m_t = max(lf_t + m_(t-1), li_t);  S_t = e^(lf_t + m_(t-1) - m_t) S_(t-1) + e^(li_t - m_t) k_t v_t^T;  n_t likewise,
+// is unrolled over a chunk of 64 tokens. With F_t the running sum of lf inside the chunk, a_s = li_s - F_s and m_0, S_0, n_0
+// what the chunk starts from:
+//     m_t = F_t + max(m_0, max_(s<=t) a_s)                                   (the same numbers as token by token)
+//     S_t = e^(F_t + m_0 - m_t) S_0 + sum_(s<=t) e^(a_s + F_t - m_t) k_s v_s^T
+// so the read-out of all 64 tokens is two matrix products, P V with P_ts = (q_t . k_s) e^(a_s + F_t - m_t) for s <= t, and
+// Q S_0 with rows weighted by e^(F_t + m_0 - m_t); n_t . q_t is the row sum of P plus the weighted n_0 . q_t; and the state
+// after the chunk is e^(F_L + m_0 - m_L) S_0 + K^T diag(e^(a_s + F_L - m_L)) V, one more product. Every exponent is <= 0.
+// Gates, maxima, weights, sums, the state and the norm of the read-out are fp32; P, the weighted values and a copy of
+// S_0 enter the products as bf16 (as the weights of attention do).
+//
+// A workgroup of four waves per (head, row of the batch) walks over the row's chunks. S^T lives in the accumulators of
+// the state product for the whole walk: wave w owns the value channels [w dv / 4, (w + 1) dv / 4). Operands are staged in
+// LDS in the layouts that v_mfma_f32_32x32x16_bf16 reads with one 16-byte load a lane: a row operand as [row][k], a
+// column operand as [column][k].
+#include "ka_common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 mc_bf16x8;
+typedef __attribute__((ext_vector_type(16))) float mc_floatx16;
+
+constexpr int MC_CHUNK = 64;
+constexpr int MC_THREADS = 256;
+constexpr int MC_PAD = 8;                   // elements a row of an LDS tile is longer than its data: spreads rows over banks
+
+struct ChunkArgs {
+    const bf16_t* q; const bf16_t* k; const bf16_t* v; const bf16_t* gate;
+    long stride;
+    const float* pre;              // fp32 [n, 2 heads]
+    float* state;                  // fp32 [state rows, heads, d dv + d + 1]
+    const int* cu_q;
+    const int* row_slot;
+    const float* gain;             // fp32 [heads dv] or null
+    bf16_t* out;
+    long out_stride;
+    int heads;
+    float q_scale, cap, eps;
+};
+
+__device__ __forceinline__ float mc_running_max(float x, int lane) {
+    for (int off = 1; off < KA_WAVE; off <<= 1) {
+        const float y = __shfl_up(x, off);
+        if (lane >= off) x = fmaxf(x, y);
+    }
+    return x;
+}
+
+// ND: d = 32 ND; NJ: dv = 128 NJ.
+template <int ND, int NJ>
+__global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkArgs a) {
+    constexpr int D = 32 * ND, DV = 128 * NJ, WJ = 32 * NJ;       // WJ: value channels a wave owns
+    constexpr int LQ = D + MC_PAD, LC = MC_CHUNK + MC_PAD;
+    extern __shared__ __attribute__((aligned(16))) unsigned char mc_lds[];
+    bf16_t* Qs = reinterpret_cast<bf16_t*>(mc_lds);               // [64][LQ]
+    bf16_t* Ks = Qs + MC_CHUNK * LQ;                              // [64][LQ]
+    bf16_t* KTs = Ks + MC_CHUNK * LQ;                             // [D][LC]
+    bf16_t* VTs = KTs + D * LC;                                   // [DV][LC]
+    bf16_t* Ps = VTs + DV * LC;                                   // [64][LC]
+    bf16_t* STs = Ps + MC_CHUNK * LC;                             // [DV][LQ]: the state the chunk starts from, transposed
+    float* fa = reinterpret_cast<float*>(STs + DV * LQ);          // a_s = li_s - F_s
+    float* fb = fa + MC_CHUNK;                                    // b_t = F_t - m_t
+    float* fm = fb + MC_CHUNK;                                    // m_t
+    float* fu = fm + MC_CHUNK;                                    // u_s = e^(a_s + b_L)
+    float* nq = fu + MC_CHUNK;                                    // n_0 . q_t (times the scale)
+    float* rowsum = nq + MC_CHUNK;                                // [2][64]: row sums of P by column block
+    float* sq = rowsum + 2 * MC_CHUNK;                            // [4][64]: sums of squares of the read-out by wave
+    float* nvec = sq + 4 * MC_CHUNK;                              // [D]: n
+    float* nnew = nvec + D;                                       // [D]
+    float* scal = nnew + D;                                       // [2]: m_0 of the next chunk, c_L
+
+    const int head = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / KA_WAVE), lane = tid % KA_WAVE;
+    const int col = lane % 32, half = lane / 32;
+    const int t0 = a.cu_q[r], t1 = a.cu_q[r + 1];
+    if (t0 >= t1) return;
+    const int slot = a.row_slot[r];
+    if (slot < 0) {
+        for (int t = t0; t < t1; ++t)
+            for (int j = tid; j < DV; j += MC_THREADS) a.out[(size_t)t * a.out_stride + head * DV + j] = (bf16_t)0.f;
+        return;
+    }
+    float* st = a.state + ((size_t)slot * a.heads + head) * (D * DV + D + 1);
+    // S^T in accumulators: tile (jb, db), register i of a lane: value channel wave WJ + jb 32 + (i / 4) 8 + half 4 + i % 4,
+    // key channel db 32 + col
+    mc_floatx16 S[NJ][ND];
+#pragma unroll
+    for (int jb = 0; jb < NJ; ++jb)
+#pragma unroll
+        for (int db = 0; db < ND; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int j = wave * WJ + jb * 32 + (i / 4) * 8 + half * 4 + i % 4, dd = db * 32 + col;
+                S[jb][db][i] = st[(size_t)dd * DV + j];
+            }
+    for (int e = tid; e < D; e += MC_THREADS) nvec[e] = st[D * DV + e];
+    float m0 = st[D * DV + D];
+
+    for (int c0 = t0; c0 < t1; c0 += MC_CHUNK) {
+        const int valid = min(MC_CHUNK, t1 - c0);
+        __syncthreads();                   // (the chunk before is done with every tile)
+        // the state the chunk starts from, as a column operand
+#pragma unroll
+        for (int jb = 0; jb < NJ; ++jb)
+#pragma unroll
+            for (int db = 0; db < ND; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int j = wave * WJ + jb * 32 + (i / 4) * 8 + half * 4 + i % 4, dd = db * 32 + col;
+                    STs[j * LQ + dd] = (bf16_t)S[jb][db][i];
+                }
+        // queries and keys as they are (rows behind the row's last token: zeros), keys and values transposed
+        for (int e = tid; e < MC_CHUNK * (D / 8); e += MC_THREADS) {
+            const int t = e / (D / 8), piece = e % (D / 8);
+            mc_bf16x8 qv, kv;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) { qv[u] = (bf16_t)0.f; kv[u] = (bf16_t)0.f; }
+            if (t < valid) {
+                const size_t at = (size_t)(c0 + t) * a.stride + head * D + piece * 8;
+                qv = *reinterpret_cast<const mc_bf16x8*>(a.q + at);
+                kv = *reinterpret_cast<const mc_bf16x8*>(a.k + at);
+            }
+            *reinterpret_cast<mc_bf16x8*>(Qs + t * LQ + piece * 8) = qv;
+            *reinterpret_cast<mc_bf16x8*>(Ks + t * LQ + piece * 8) = kv;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) KTs[(piece * 8 + u) * LC + t] = kv[u];
+        }
+        for (int e = tid; e < MC_CHUNK * (DV / 8); e += MC_THREADS) {
+            const int t = e / (DV / 8), piece = e % (DV / 8);
+            mc_bf16x8 vv;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) vv[u] = (bf16_t)0.f;
+            if (t < valid) vv = *reinterpret_cast<const mc_bf16x8*>(a.v + (size_t)(c0 + t) * a.stride + head * DV + piece * 8);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) VTs[(piece * 8 + u) * LC + t] = vv[u];
+        }
+        // the gates of the chunk: one wave, a token a lane
+        if (wave == 0) {
+            float li = -INFINITY, lf = 0.f;              // (behind the last token: no input, nothing forgotten)
+            if (lane < valid) {
+                const size_t at = (size_t)(c0 + lane) * 2 * a.heads;
+                li = a.cap * tanhf(a.pre[at + head] / a.cap);
+                const float z = a.cap * tanhf(a.pre[at + a.heads + head] / a.cap);
+                lf = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+            }
+            const float F = ka_wave_running_sum(lf);
+            const float as = li - F;
+            const float top = fmaxf(m0, mc_running_max(as, lane));
+            fa[lane] = as;
+            fb[lane] = -top;                             // F_t - m_t with m_t = F_t + top
+            fm[lane] = F + top;
+            const float b_last = -ka_lane_value(top, KA_WAVE - 1);
+            fu[lane] = expf(as + b_last);
+            if (lane == 0) {
+                scal[0] = ka_lane_value(F + top, KA_WAVE - 1);
+                scal[1] = expf(m0 + b_last);
+            }
+        }
+        __syncthreads();
+        // n_0 . q_t, a token a thread
+        if (tid < MC_CHUNK) {
+            float acc = 0.f;
+            for (int dd = 0; dd < D; ++dd) acc += nvec[dd] * (float)Qs[tid * LQ + dd];
+            nq[tid] = acc * a.q_scale;
+        }
+        // scores of the chunk against itself: wave w computes the block of tokens tb = w / 2 against keys sb = w % 2
+        {
+            const int tb = wave / 2, sb = wave % 2;
+            mc_floatx16 g;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) g[i] = 0.f;
+            // (rows are queries, columns keys: a lane holds 16 queries' scores against ONE key)
+#pragma unroll
+            for (int kk = 0; kk < D / 16; ++kk) {
+                const mc_bf16x8 qa = *reinterpret_cast<const mc_bf16x8*>(Qs + (tb * 32 + col) * LQ + kk * 16 + half * 8);
+                const mc_bf16x8 kb = *reinterpret_cast<const mc_bf16x8*>(Ks + (sb * 32 + col) * LQ + kk * 16 + half * 8);
+                g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kb, g, 0, 0, 0);
+            }
+            const int s = sb * 32 + col;
+            const float a_s = fa[s];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int t = tb * 32 + (i / 4) * 8 + half * 4 + i % 4;
+                const float p = s <= t ? g[i] * a.q_scale * expf(a_s + fb[t]) : 0.f;
+                Ps[t * LC + s] = (bf16_t)p;
+                const float sum = ka_lanes_reduce<1, 32>(p, KaSum{});
+                if (col == 0) rowsum[sb * MC_CHUNK + t] = sum;
+            }
+        }
+        __syncthreads();
+        // read-out: O = P V + diag(e^(m_0 + b_t)) scale Q S_0, the wave's value channels of all 64 tokens
+        mc_floatx16 O[2][NJ];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int jb = 0; jb < NJ; ++jb) {
+                mc_floatx16 carry;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) carry[i] = 0.f;
+#pragma unroll
+                for (int kk = 0; kk < D / 16; ++kk) {
+                    const mc_bf16x8 qa = *reinterpret_cast<const mc_bf16x8*>(Qs + (tb * 32 + col) * LQ + kk * 16 + half * 8);
+                    const mc_bf16x8 sb = *reinterpret_cast<const mc_bf16x8*>(STs + (wave * WJ + jb * 32 + col) * LQ + kk * 16 + half * 8);
+                    carry = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, sb, carry, 0, 0, 0);
+                }
+                mc_floatx16 acc;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int t = tb * 32 + (i / 4) * 8 + half * 4 + i % 4;
+                    acc[i] = carry[i] * a.q_scale * expf(m0 + fb[t]);
+                }
+#pragma unroll
+                for (int kk = 0; kk < MC_CHUNK / 16; ++kk) {
+                    const mc_bf16x8 pa = *reinterpret_cast<const mc_bf16x8*>(Ps + (tb * 32 + col) * LC + kk * 16 + half * 8);
+                    const mc_bf16x8 vb = *reinterpret_cast<const mc_bf16x8*>(VTs + (wave * WJ + jb * 32 + col) * LC + kk * 16 + half * 8);
+                    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(pa, vb, acc, 0, 0, 0);
+                }
+                O[tb][jb] = acc;
+            }
+        // divided by max(|n_t . q_t|, e^(-m_t)) + 1e-6, then this wave's share of every token's sum of squares
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int t = tb * 32 + (i / 4) * 8 + half * 4 + i % 4;
+                const float dot = expf(m0 + fb[t]) * nq[t] + (rowsum[t] + rowsum[MC_CHUNK + t]);
+                const float den = fmaxf(fabsf(dot), expf(-fm[t])) + 1e-6f;
+                float ssq = 0.f;
+#pragma unroll
+                for (int jb = 0; jb < NJ; ++jb) {
+                    O[tb][jb][i] /= den;
+                    ssq += O[tb][jb][i] * O[tb][jb][i];
+                }
+                ssq = ka_lanes_reduce<1, 32>(ssq, KaSum{});
+                if (col == 0) sq[wave * MC_CHUNK + t] = ssq;
+            }
+        __syncthreads();
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int t = tb * 32 + (i / 4) * 8 + half * 4 + i % 4;
+                if (t < valid) {
+                    const float total = (sq[t] + sq[MC_CHUNK + t]) + (sq[2 * MC_CHUNK + t] + sq[3 * MC_CHUNK + t]);
+                    const float rr = 1.0f / sqrtf(total / (float)DV + a.eps);
+#pragma unroll
+                    for (int jb = 0; jb < NJ; ++jb) {
+                        const int c = head * DV + wave * WJ + jb * 32 + col;
+                        const size_t tok = (size_t)(c0 + t);
+                        const float g = a.gate ? 1.0f / (1.0f + expf(-(float)a.gate[tok * a.stride + c])) : 1.f;
+                        a.out[tok * a.out_stride + c] = (bf16_t)(O[tb][jb][i] * rr * (a.gain ? a.gain[c] : 1.f) * g);
+                    }
+                }
+            }
+        // the state after the chunk: S^T <- c_L S^T + (diag(u) V)^T K, n <- c_L n + K^T u
+        const float c_last = scal[1];
+        if (tid < D) {
+            float acc = c_last * nvec[tid];
+            for (int s = 0; s < MC_CHUNK; ++s) acc += fu[s] * (float)KTs[tid * LC + s];
+            nnew[tid] = acc;
+        }
+#pragma unroll
+        for (int jb = 0; jb < NJ; ++jb) {
+#pragma unroll
+            for (int db = 0; db < ND; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) S[jb][db][i] *= c_last;
+#pragma unroll
+            for (int kk = 0; kk < MC_CHUNK / 16; ++kk) {
+                const int s0 = kk * 16 + half * 8;
+                const mc_bf16x8 vraw = *reinterpret_cast<const mc_bf16x8*>(VTs + (wave * WJ + jb * 32 + col) * LC + s0);
+                mc_bf16x8 va;
+#pragma unroll
+                for (int u = 0; u < 8; ++u) va[u] = (bf16_t)((float)vraw[u] * fu[s0 + u]);
+#pragma unroll
+                for (int db = 0; db < ND; ++db) {
+                    const mc_bf16x8 kb = *reinterpret_cast<const mc_bf16x8*>(KTs + (db * 32 + col) * LC + s0);
+                    S[jb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va, kb, S[jb][db], 0, 0, 0);
+                }
+            }
+        }
+        m0 = scal[0];
+        __syncthreads();
+        if (tid < D) nvec[tid] = nnew[tid];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int jb = 0; jb < NJ; ++jb)
+#pragma unroll
+        for (int db = 0; db < ND; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int j = wave * WJ + jb * 32 + (i / 4) * 8 + half * 4 + i % 4, dd = db * 32 + col;
+                st[(size_t)dd * DV + j] = S[jb][db][i];
+            }
+    for (int e = tid; e < D; e += MC_THREADS) st[D * DV + e] = nvec[e];
+    if (tid == 0) st[D * DV + D] = m0;
+}
+
+template <int ND, int NJ>
+static size_t mc_lds_bytes() {
+    constexpr int D = 32 * ND, DV = 128 * NJ, LQ = D + MC_PAD, LC = MC_CHUNK + MC_PAD;
+    return sizeof(bf16_t) * ((size_t)2 * MC_CHUNK * LQ + (size_t)D * LC + (size_t)DV * LC + (size_t)MC_CHUNK * LC + (size_t)DV * LQ)
+        + sizeof(float) * (5 * MC_CHUNK + 2 * MC_CHUNK + 4 * MC_CHUNK + 2 * D + 2);
+}
+
+// Whether the kernel covers heads of these sizes: keys of 32, 64 or 128 channels, values of 128 or 256 (128 x 256: its
+// tiles do not fit in LDS).
+KA_API int ka_matrix_memory_chunks_supported(int d, int dv) {
+    return (d == 32 || d == 64 || d == 128) && (dv == 128 || dv == 256) && !(d == 128 && dv == 256) ? 1 : 0;
+}
+
+KA_API int ka_matrix_memory_chunks_bf16(const void* q, const void* k, const void* v, const void* gate, long stride,
+                                        const float* pre, float* state, const int* cu_q, const int* row_slot,
+                                        const float* gain, void* out, long out_stride, int n_rows, int heads, int d, int dv,
+                                        float q_scale, float cap, float eps, hipStream_t stream) {
+    const char* who = "ka_matrix_memory_chunks_bf16";
+    KA_CHECK(n_rows >= 0 && heads > 0 && ka_matrix_memory_chunks_supported(d, dv), "%s: heads of %d x %d not covered", who, d, dv);
+    KA_CHECK(cap > 0.f && eps >= 0.f, "%s: the gates' cap must be positive", who);
+    KA_CHECK(heads <= 65535 && n_rows <= 65535, "%s: too many heads or rows", who);
+    KA_CHECK((uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 && stride % 8 == 0,
+             "%s: operands must be 16-byte aligned", who);
+    if (n_rows == 0) return 0;
+    ChunkArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)gate, stride, pre, state, cu_q, row_slot,
+                gain, (bf16_t*)out, out_stride, heads, q_scale, cap, eps};
+    const dim3 grid(heads, n_rows), block(MC_THREADS);
+#define MC_LAUNCH(ND, NJ)                                                                                                   \
+    if (d == 32 * ND && dv == 128 * NJ) {                                                                                   \
+        static bool sized = false;                                                                                          \
+        if (!sized) {                                                                                                       \
+            (void)hipFuncSetAttribute((const void*)matrix_memory_chunk_kernel<ND, NJ>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            sized = true;                                                                                                   \
+        }                                                                                                                   \
+        const size_t lds = mc_lds_bytes<ND, NJ>();                                                                          \
+        hipLaunchKernelGGL((matrix_memory_chunk_kernel<ND, NJ>), grid, block, lds, stream, a);                              \
+    }
+    MC_LAUNCH(1, 1) MC_LAUNCH(2, 1) MC_LAUNCH(4, 1) MC_LAUNCH(1, 2) MC_LAUNCH(2, 2)
+#undef MC_LAUNCH
+    KA_LAUNCH_CHECK();
+    return 0;
+}

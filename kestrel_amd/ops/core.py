@@ -417,14 +417,15 @@ def branches_sum(x: torch.Tensor, a: torch.Tensor, gain_a: Optional[torch.Tensor
 
 def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
                   row_slot: torch.Tensor, gain: Optional[torch.Tensor], out: torch.Tensor, n_heads: int, head_dim: int,
-                  value_dim: int, q_scale: float, cap: float, eps: float, single_tokens: bool) -> None:
+                  value_dim: int, q_scale: float, cap: float, eps: float, single_tokens: bool, chunks: bool = False) -> None:
     """The gated matrix memory over the packed tokens of a step. ``projected`` ``[n, *]`` holds queries, keys, values and
     (optionally) the output gate's pre-activations at the column ``offsets = (q, k, v, gate or None)``; ``pre`` fp32
     ``[n, 2 heads]`` the pre-activations of the input gates, then of the forget gates; ``state`` fp32
     ``[slots + 1, heads * (hd * hdv + hd + 1)]`` (per head the matrix, the normaliser and the running maximum), advanced in
     place for row ``r`` at ``row_slot[r]`` over its tokens ``cu_q[r] .. cu_q[r + 1]`` (a negative slot: zeros are written,
     no state is touched). ``out`` ``[n, heads * hdv]``: every head's read-out divided by its root mean square, times ``gain``
-    (fp32 ``[heads * hdv]``), times the sigmoid of the gate."""
+    (fp32 ``[heads * hdv]``), times the sigmoid of the gate. ``chunks``: bf16 prompt portions go to the matrix-core kernel that
+    unrolls the recurrence over chunks of 64 tokens, where it covers the sizes (``ops.fast.matrix_memory_chunks_bf16``)."""
     _dev(projected, pre, state, cu_q, row_slot, gain, out)
     n = projected.shape[0]
     n_rows = row_slot.numel()
@@ -441,6 +442,11 @@ def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: to
     _need(out.dtype == projected.dtype and out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * value_dim),
           "matrix_memory: out must be [n, heads hdv] of the projected type")
     _need(gain is None or (gain.dtype == torch.float32 and gain.numel() == n_heads * value_dim), "matrix_memory: gain fp32 [heads hdv]")
+    if chunks and projected.dtype == torch.bfloat16 and not single_tokens:
+        from . import fast
+        if fast.matrix_memory_chunks_bf16(projected, offsets, pre, state, cu_q, row_slot, gain, out, n_heads, head_dim, value_dim,
+                                          q_scale, cap, eps):
+            return
     size = projected.element_size()
     base = projected.data_ptr()
     stride = projected.stride(0) if n > 1 else width

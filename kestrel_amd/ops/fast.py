@@ -55,6 +55,9 @@ _SIGNATURES = {
     "ka_attention_biased_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p],
+    "ka_matrix_memory_chunks_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
+                                     _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
+                                     _c_void_p],
     "ka_linear_skinny_norm_store": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p,
                                     _c_int, _c_long, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
 }
@@ -642,4 +645,28 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         _ptr(positions), _ptr(slopes), out.data_ptr(), out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim,
         value_dim, page_size, waves, int(sink is not None), float(sink or 0.0), _ptr(bias_table),
         int(bias_table.shape[1]) if bias_table is not None else 0, stream_ptr()))
+    return True
+
+
+def matrix_memory_chunks_bf16(projected, offsets, pre, state, cu_q, row_slot, gain, out, n_heads, head_dim, value_dim,
+                              q_scale, cap, eps) -> bool:
+    """``ops.core.matrix_memory`` for prompt portions on the matrix cores: the recurrence unrolled over chunks of 64 tokens
+    (operands as for ``ops.core.matrix_memory``, which has checked them). False: head sizes or alignment not covered,
+    nothing was run."""
+    handle = lib()
+    n = projected.shape[0]
+    if n == 0:
+        return True
+    if projected.dtype != torch.bfloat16 or not handle.ka_matrix_memory_chunks_supported(int(head_dim), int(value_dim)):
+        return False
+    oq, ok, ov, og = offsets
+    size, base = projected.element_size(), projected.data_ptr()
+    stride = projected.stride(0) if n > 1 else projected.shape[1]
+    if base % 16 or stride % 8 or any(o % 8 for o in (oq, ok, ov)) or (n_heads * head_dim) % 8:
+        return False
+    _check(handle.ka_matrix_memory_chunks_bf16(base + oq * size, base + ok * size, base + ov * size,
+                                               None if og is None else base + og * size, stride, pre.data_ptr(), state.data_ptr(),
+                                               cu_q.data_ptr(), row_slot.data_ptr(), _ptr(gain), out.data_ptr(),
+                                               out.stride(0) if n > 1 else n_heads * value_dim, int(row_slot.numel()), n_heads,
+                                               head_dim, value_dim, float(q_scale), float(cap), float(eps), stream_ptr()))
     return True

@@ -28,7 +28,9 @@ class MatrixMemory(Mixer):
 
     One launch projects q | k | v | gate in the activation type; the two gates' pre-activations come from a linear of their
     own with fp32 output (what enters the recurrence stays in 32 bits); one kernel then walks over every row's tokens in
-    order (``ops.core.matrix_memory``), whatever the step holds: a prompt, a portion, single tokens. Rows without a
+    order (``ops.core.matrix_memory``), whatever the step holds: a prompt, a portion, single tokens. In bf16, steps that
+    hold more than single tokens go to a kernel that unrolls the recurrence over chunks of 64 tokens into products on the
+    matrix cores, where it covers the head sizes. Rows without a
     request (the padding of a replayed step) write zeros and touch no state."""
 
     replays_every_step = True
@@ -82,7 +84,7 @@ class MatrixMemory(Mixer):
         offsets = (0, self.qk_dim, 2 * self.qk_dim, 2 * self.qk_dim + self.v_dim if self.gated else None)
         core.matrix_memory(projected, offsets, pre, cache.state, batch.cu_q, batch.row_slot, self.gain, out, spec.n_heads,
                            spec.head_dim, spec.value_dim, float(spec.head_dim) ** -0.5, spec.gate_cap, spec.eps,
-                           single_tokens=batch.max_q == 1)
+                           single_tokens=bool(batch.decode_only), chunks=True)
         return out
 
     def output_projection(self):

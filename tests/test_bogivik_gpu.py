@@ -433,15 +433,18 @@ def test_gate_and_branches_kernels(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
-@pytest.mark.parametrize("heads, d, dv", [(3, 20, 36), (1, 8, 300), (2, 64, 64), (2, 200, 200)])
+@pytest.mark.parametrize("heads, d, dv", [(3, 20, 36), (1, 8, 300), (2, 64, 64), (2, 200, 200), (2, 64, 128), (1, 32, 256),
+                                          (1, 128, 128), (3, 64, 256)])
 def test_matrix_memory_kernel(heads, d, dv, dtype):
     """Rows of unequal lengths in one launch, cut into steps (a prompt, portions, single tokens), against the plain
     recurrence over the whole sequence: the state in its slot carries everything; a row without a request writes zeros;
-    large gates stay finite through the running maximum. (200 x 200: a state too large for LDS.)"""
+    large gates stay finite through the running maximum. (200 x 200: a state too large for LDS; value heads of 128 and
+    256: in bf16 the portions go through the kernel that unrolls the recurrence over chunks of 64 tokens, here with rows
+    of less than a chunk, of several chunks and a part, and a state that single tokens have advanced in between.)"""
     from kestrel_amd.ops import core
 
     g = _gen(4)
-    lengths = [37, 5, 1, 20]
+    lengths = [150, 5, 1, 90]
     cap, eps, scale = 6.0, 1e-5, d ** -0.5
     width = 2 * heads * d + 2 * heads * dv + 5
     data = {r: dict(x=(torch.randn(L, width, generator=g)).to(dtype), pre=torch.randn(L, 2 * heads, generator=g) * 8 + 1.0)
@@ -467,7 +470,7 @@ def test_matrix_memory_kernel(heads, d, dv, dtype):
         return plain.rms_norm(o, None, eps).reshape(L, heads * dv) * gain.double() * torch.sigmoid(gate)
 
     # steps: (row, tokens) lists; rows 0 and 3 in portions and single tokens, a padding row (slot -1) in the middle
-    steps = [[(0, 10), (1, 5)], [(0, 1), (None, 3), (2, 1), (3, 2)], [(0, 1), (3, 1)], [(0, 25), (3, 17)]]
+    steps = [[(0, 10), (1, 5)], [(0, 1), (None, 3), (2, 1), (3, 2)], [(0, 1), (3, 1)], [(0, 138), (3, 87)]]
     done = {r: 0 for r in data}
     got = {r: [] for r in data}
     for step in steps:
@@ -486,7 +489,7 @@ def test_matrix_memory_kernel(heads, d, dv, dtype):
         out = torch.full((x.shape[0], heads * dv), 7.0, dtype=dtype, device=DEV)
         core.matrix_memory(x, offsets, torch.cat(pres).to(DEV).contiguous(), state, torch.tensor(cu, dtype=torch.int32, device=DEV),
                            torch.tensor(slots, dtype=torch.int32, device=DEV), gain.to(DEV), out, heads, d, dv, scale, cap, eps,
-                           single_tokens=all(count == 1 for _, count in step))
+                           single_tokens=all(count == 1 for _, count in step), chunks=True)
         for i, (r, count) in enumerate(step):
             piece = out[cu[i]:cu[i + 1]].double().cpu()
             if r is None:
