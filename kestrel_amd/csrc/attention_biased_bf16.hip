@@ -59,7 +59,8 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo, const int* __restrict__ kv_hi,
                    const int* __restrict__ positions, const float* __restrict__ slopes, bf16_t* __restrict__ out,
                    long out_row_stride, float scale, int H, int Hkv, int hdv, int heads_per_block, int has_sink,
-                   float sink_score, const float* __restrict__ bias_table, int bias_len) {
+                   float sink_score, const float* __restrict__ bias_table, int bias_len, const bf16_t* __restrict__ gate,
+                   long gate_row_stride) {
     constexpr int HD = NK * 16;
     constexpr int REC = 16 * NV + 2;            // floats a lane hands over at a merge: its outputs, m and l
     extern __shared__ float mrg[];              // [waves / 2][REC][64]
@@ -267,6 +268,17 @@ attn_biased_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const float inv = l > 0.f ? 1.0f / l : 0.f;
     // register i of block b: channel b * 32 + (i / 4) * 8 + half * 4 + i % 4 of the lane's column
     bf16_t* op = out + (size_t)tok * out_row_stride + (size_t)head * hdv;
+    if (gate) {
+        // an output gate: every channel times the sigmoid of the gate's pre-activation of the same token and channel
+        const bf16_t* gp = gate + (size_t)tok * gate_row_stride + (size_t)head * hdv;
+#pragma unroll
+        for (int b = 0; b < NV; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int ch = b * 32 + (i / 4) * 8 + half * 4 + i % 4;
+                if (ch < hdv) o[b][i] *= 1.0f / (1.0f + __expf(-(float)gp[ch]));
+            }
+    }
 #pragma unroll
     for (int b = 0; b < NV; ++b)
 #pragma unroll
@@ -306,7 +318,7 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
                                     const int* kv_hi, const int* positions, const float* slopes, void* out,
                                     long out_row_stride, float scale, int n, int H, int Hkv, int hd, int hdv,
                                     int page_size, int waves, int has_sink, float sink_score, const float* bias_table,
-                                    int bias_len, hipStream_t stream) {
+                                    int bias_len, const void* gate, long gate_row_stride, hipStream_t stream) {
     const char* who = "ka_attention_biased_bf16";
     KA_CHECK(n >= 0 && n_blocks >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes", who);
     KA_CHECK(page_size == AB_PAGE && ab_sizes_covered(hd, hdv), "%s: head sizes %d / %d or page size %d not covered", who, hd, hdv, page_size);
@@ -343,7 +355,8 @@ KA_API int ka_attention_biased_bf16(const void* q, long q_row_stride, const void
         hipLaunchKernelGGL((attn_biased_kernel<NK, NV>), grid, dim3(KA_WAVE * waves), lds, stream, (const bf16_t*)q,       \
                            q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, \
                            qblk_tok, cu_q, token_row, kv_lo, kv_hi, positions, slopes, (bf16_t*)out, out_row_stride, scale, \
-                           H, Hkv, hdv, heads_per_block, has_sink, sink_score, bias_table, bias_len);                      \
+                           H, Hkv, hdv, heads_per_block, has_sink, sink_score, bias_table, bias_len, (const bf16_t*)gate, \
+                           gate_row_stride);                                                                               \
     }
 #define AB_LAUNCH_NK(NK) AB_LAUNCH(NK, 1) AB_LAUNCH(NK, 2) AB_LAUNCH(NK, 3) AB_LAUNCH(NK, 4)
     AB_LAUNCH_NK(2) AB_LAUNCH_NK(3) AB_LAUNCH_NK(4) AB_LAUNCH_NK(6) AB_LAUNCH_NK(8)

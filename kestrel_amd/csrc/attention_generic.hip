@@ -16,6 +16,8 @@
 //    of query position i against key position j is lowered by slopes[h] * (i - j);
 //  * a distance table (fp32 [H, bias_len]) with positions: the score of query position i against key position j is
 //    raised by table[h, min(i - j, bias_len - 1)] (a learned bias per head and distance, constant from some distance on);
+//  * an output gate (rows of the activation type, [n, H hdv] with a row stride of their own): the output is multiplied
+//    element by element by the sigmoid of it;
 //  * a sink: one more term exp(sink_score) in the softmax's denominator that carries no value
 //    (has_sink != 0). The running maximum and sum then start from that term instead of from nothing.
 #include "ka_common.h"
@@ -40,7 +42,8 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
                          T* __restrict__ out, long out_row_stride, float scale, int H, int Hkv,
                          int hd, int hdv, int page_size, const int* __restrict__ positions,
                          const float* __restrict__ slopes, int has_sink, float sink_score,
-                         const float* __restrict__ bias_table, int bias_len) {
+                         const float* __restrict__ bias_table, int bias_len, const T* __restrict__ gate,
+                         long gate_row_stride) {
     __shared__ float qs[ATT_MAX_HD];
     __shared__ float ps[KA_WAVE];
     __shared__ long offs[KA_WAVE];   // value cache offset of channel 0 of each key of the chunk
@@ -123,7 +126,12 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
 #pragma unroll
     for (int i = 0; i < ATT_MAX_HD / KA_WAVE; ++i) {
         int d = lane + i * KA_WAVE;
-        if (d < hdv) op[d] = ka_from_float<T>(o[i] * inv);
+        if (d < hdv) {
+            float y = o[i] * inv;
+            // (an output gate: the head's channels times the sigmoid of the gate's pre-activations of the same token)
+            if (gate) y *= 1.0f / (1.0f + expf(-ka_to_float(gate[(size_t)t * gate_row_stride + (size_t)h * hdv + d])));
+            op[d] = ka_from_float<T>(y);
+        }
     }
 }
 
@@ -133,7 +141,7 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
                                 long out_row_stride, float scale, int n, int H, int Hkv, int hd,
                                 int page_size, int hdv, const int* positions, const float* slopes,
                                 int has_sink, float sink_score, const float* bias_table, int bias_len,
-                                hipStream_t stream) {
+                                const void* gate, long gate_row_stride, hipStream_t stream) {
     KA_CHECK(bias_table == nullptr || (positions != nullptr && bias_len > 0), "ka_attention_generic: a distance table needs the queries' positions");
     KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0 && hdv > 0, "ka_attention_generic: bad sizes");
     KA_CHECK(hdv <= ATT_MAX_HD, "ka_attention_generic: value size %d above %d", hdv, ATT_MAX_HD);
@@ -148,12 +156,12 @@ KA_API int ka_attention_generic(const void* q, int dtype, long q_row_stride, con
         hipLaunchKernelGGL(attention_generic_kernel<float>, grid, block, 0, stream, (const float*)q, q_row_stride,
                            (const float*)k_cache, (const float*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (float*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score, bias_table, bias_len);
+                           sink_score, bias_table, bias_len, (const float*)gate, gate_row_stride);
     else if (dtype == KA_BF16)
         hipLaunchKernelGGL(attention_generic_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
                            (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
                            kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, hd, hdv, page_size, positions, slopes, has_sink,
-                           sink_score, bias_table, bias_len);
+                           sink_score, bias_table, bias_len, (const bf16_t*)gate, gate_row_stride);
     else
         KA_CHECK(false, "ka_attention_generic: unsupported dtype %d", dtype);
     KA_LAUNCH_CHECK();

@@ -345,7 +345,21 @@ __global__ void __launch_bounds__(MP_THREADS) matrix_memory_kernel(MemoryArgs a)
             const int j = idx % dv, p = idx / dv;
             const float vj = take * vs[j];
             float acc = 0.f;
-            for (int i = p; i < d; i += parts) {
+            // eight numbers of the state in flight at a time (a load behind a store to the same array would wait for it)
+            int i = p;
+            for (; i + 7 * parts < d; i += 8 * parts) {
+                float s8[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s8[u] = S[(size_t)(i + u * parts) * dv + j];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    s8[u] = keep * s8[u] + ks[i + u * parts] * vj;
+                    acc += s8[u] * qs[i + u * parts];
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) S[(size_t)(i + u * parts) * dv + j] = s8[u];
+            }
+            for (; i < d; i += parts) {
                 const float s = keep * S[(size_t)i * dv + j] + ks[i] * vj;
                 S[(size_t)i * dv + j] = s;
                 acc += s * qs[i];

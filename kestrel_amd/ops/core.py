@@ -31,7 +31,7 @@ _SIGNATURES = {
                           _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                              _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
-                             _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_int, _c_void_p],
+                             _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_rmsnorm": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
     "ka_qkv_prepare": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_float, _c_int,
@@ -513,14 +513,15 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       out: torch.Tensor, scale: float, n_heads: int, n_kv_heads: int, head_dim: int,
                       value_dim: Optional[int] = None, positions: Optional[torch.Tensor] = None,
                       slopes: Optional[torch.Tensor] = None, sink: Optional[float] = None,
-                      bias_table: Optional[torch.Tensor] = None) -> None:
+                      bias_table: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
     """Paged attention of ``n`` packed tokens; ``q`` may be a strided view into a qkv buffer.
 
     ``value_dim``: size of a value head where it differs from ``head_dim`` (``out`` is ``[n, H value_dim]``).
     ``slopes`` (fp32 ``[H]``) with ``positions`` (int32 ``[n]``): the score of a query at place ``i`` against the key
     at place ``j`` is lowered by ``slopes[h] * (i - j)``. ``sink``: the score of one more term of the softmax's
     denominator that carries no value (``None``: no such term). ``bias_table`` (fp32 ``[H, T]``) with ``positions``: the
-    score is raised by ``bias_table[h, min(i - j, T - 1)]``."""
+    score is raised by ``bias_table[h, min(i - j, T - 1)]``. ``gate`` (``[n, H value_dim]`` of the q type, rows may lie in a
+    wider buffer): the output is multiplied element by element by ``sigmoid(gate)``."""
     _dev(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, positions, slopes, bias_table)
     n = q.shape[0]
     value_dim = head_dim if value_dim is None else int(value_dim)
@@ -539,6 +540,8 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
               and bias_table.is_contiguous(), "attention: the distance table must be contiguous fp32 [H, T]")
         _need(positions is not None and positions.dtype == torch.int32 and positions.numel() == n and positions.is_contiguous(),
               "attention: a distance table needs the queries' positions, int32 [n]")
+    _need(gate is None or (gate.is_cuda and gate.dtype == q.dtype and gate.dim() == 2 and gate.stride(1) == 1
+                           and tuple(gate.shape) == (n, n_heads * value_dim)), "attention: the gate must be [n, H hdv] of the q type")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "attention: block table must be contiguous int32 [rows, pages]")
     for t in (token_row, kv_hi) + ((kv_lo,) if kv_lo is not None else ()):
@@ -549,7 +552,8 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                                       out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size,
                                       value_dim, _ptr(positions) if (slopes is not None or bias_table is not None) else None,
                                       _ptr(slopes), int(sink is not None), float(sink or 0.0), _ptr(bias_table),
-                                      int(bias_table.shape[1]) if bias_table is not None else 0, stream_ptr()))
+                                      int(bias_table.shape[1]) if bias_table is not None else 0, _ptr(gate),
+                                      (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0, stream_ptr()))
 
 
 def _pending_args(who: str, rows: int, pending, pending_at):

@@ -54,7 +54,7 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],      # W, ldw, bias, out, ..., stream
     "ka_attention_biased_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_int,
                                  _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
-                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_matrix_memory_chunks_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                      _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
                                      _c_void_p],
@@ -601,7 +601,7 @@ def biased_query_block(head_dim: int, value_dim: int) -> Optional[int]:
 
 
 def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
-                          head_dim, value_dim, positions, slopes, sink, batch, bias_table=None) -> bool:
+                          head_dim, value_dim, positions, slopes, sink, batch, bias_table=None, gate=None) -> bool:
     """Attention with the further terms of ``ops.core.attention_generic`` (values of ``value_dim`` channels, ``slopes``
     times the distance taken off the scores, a ``sink`` in the softmax's denominator) on the matrix cores, for prompt
     portions, mixed steps and decode steps alike. False: not covered (head sizes, page size, alignment, no list of
@@ -618,6 +618,9 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         return False
     if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or positions is None):
         raise KernelError("attention: slopes must be fp32 [H] and come with the queries' positions")
+    if gate is not None and (gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.stride(1) != 1
+                             or tuple(gate.shape) != (n, n_heads * value_dim)):
+        raise KernelError("attention: the output gate must be bf16 [n, H hdv]")
     if bias_table is not None and (bias_table.dtype != torch.float32 or bias_table.dim() != 2 or bias_table.shape[0] != n_heads
                                    or not bias_table.is_contiguous() or positions is None):
         raise KernelError("attention: the distance table must be contiguous fp32 [H, T] and come with the queries' positions")
@@ -644,7 +647,8 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         _ptr(rows), _ptr(first), n_blocks, batch.cu_q.data_ptr(), token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(),
         _ptr(positions), _ptr(slopes), out.data_ptr(), out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim,
         value_dim, page_size, waves, int(sink is not None), float(sink or 0.0), _ptr(bias_table),
-        int(bias_table.shape[1]) if bias_table is not None else 0, stream_ptr()))
+        int(bias_table.shape[1]) if bias_table is not None else 0, _ptr(gate),
+        (gate.stride(0) if n > 1 else n_heads * value_dim) if gate is not None else 0, stream_ptr()))
     return True
 
 

@@ -293,13 +293,15 @@ class PagedAttention(Mixer):
                          float(norm.eps) if norm is not None else 0.0, self._freqs, self._pairing,
                          (self.growth.coef, self.growth.every) if self.growth is not None else None,
                          self.blend.role if self.blend is not None else None, other, self._blend_weight)
-        done = False
+        gate = projected[:, self.qkv_dim:] if self.gated else None
+        done = gated = False          # (gated: the attention kernel has applied the output gate in its epilogue)
         if qkv.dtype == torch.bfloat16:
             from ..ops import fast
             if self.extended:
-                done = fast.attention_biased_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo,
-                                                  batch.kv_hi, out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim,
-                                                  self.value_dim, batch.positions, None, None, batch, bias_table=self._bias_table)
+                done = gated = fast.attention_biased_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo,
+                                                          batch.kv_hi, out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim,
+                                                          self.value_dim, batch.positions, None, None, batch,
+                                                          bias_table=self._bias_table, gate=gate)
             else:
                 paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                                 self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
@@ -307,9 +309,10 @@ class PagedAttention(Mixer):
         if not done:
             core.attention_generic(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                                    self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, self.value_dim, batch.positions,
-                                   None, None, bias_table=self._bias_table)
-        if self.gated:
-            core.gate_mul(out, projected[:, self.qkv_dim:])
+                                   None, None, bias_table=self._bias_table, gate=gate)
+            gated = True
+        if self.gated and not gated:
+            core.gate_mul(out, gate)
         return out
 
     @staticmethod

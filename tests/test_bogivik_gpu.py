@@ -546,13 +546,17 @@ def test_attention_with_a_distance_table(hd, hdv, G, H, dtype):
                                  ([100 + i for i in range(33)], [96] * 28 + [128] * 5, False), ([19], [16], True)):
         n = len(places)
         queries = torch.randn(n, H * hd, generator=g).to(dtype)
+        # (an output gate, applied in the kernels' epilogues, on every second case; its rows lie in a wider buffer)
+        gate = (torch.randn(n, H * hdv + 8, generator=g) * 2).to(dtype).to(DEV)[:, 8:] if len(places) % 2 else None
         want = want_for(places, lows)
+        if gate is not None:
+            want = want * torch.sigmoid(gate.double().cpu())
         args = dict(token_row=torch.zeros(n, dtype=torch.int32, device=DEV), kv_lo=torch.tensor(lows, dtype=torch.int32, device=DEV),
                     kv_hi=torch.tensor([p + 1 for p in places], dtype=torch.int32, device=DEV))
         pos = torch.tensor(places, dtype=torch.int32, device=DEV)
         out = torch.zeros(n, H * hdv, dtype=dtype, device=DEV)
         core.attention_generic(queries.to(DEV), k_cache, v_cache, block_table, args["token_row"], args["kv_lo"], args["kv_hi"], out,
-                               scale, H, G, hd, hdv, pos, None, None, bias_table=table.to(DEV))
+                               scale, H, G, hd, hdv, pos, None, None, bias_table=table.to(DEV), gate=gate)
         assert torch.allclose(out.double().cpu(), want, **_tol(dtype)), f"generic kernel, places {places[0]}.."
         if dtype == torch.bfloat16 and fast.biased_query_block(hd, hdv):
             from types import SimpleNamespace
@@ -563,5 +567,6 @@ def test_attention_with_a_distance_table(hd, hdv, G, H, dtype):
                                                          torch.tensor(firsts, dtype=torch.int32, device=DEV))})
             out = torch.zeros(n, H * hdv, dtype=dtype, device=DEV)
             assert fast.attention_biased_bf16(queries.to(DEV), k_cache, v_cache, block_table, args["token_row"], args["kv_lo"],
-                                              args["kv_hi"], out, scale, H, G, hd, hdv, pos, None, None, batch, bias_table=table.to(DEV))
+                                              args["kv_hi"], out, scale, H, G, hd, hdv, pos, None, None, batch, bias_table=table.to(DEV),
+                                              gate=gate)
             assert torch.allclose(out.double().cpu(), want, **_tol(dtype)), f"matrix-core kernel, places {places[0]}.."
