@@ -104,13 +104,14 @@ class _Group:
 
 
 class _SlotState:
-    __slots__ = ("tables", "length", "quota", "first_page")
+    __slots__ = ("tables", "length", "quota", "first_page", "held")
 
     def __init__(self, n_groups: int) -> None:
         self.tables: List[List[int]] = [[] for _ in range(n_groups)]   # -1 = given back
         self.length = 0                                                 # positions backed so far
         self.quota: List[int] = [0] * n_groups                          # pages promised at admission
         self.first_page: List[int] = [0] * n_groups                     # logical pages below it are given back
+        self.held: List[int] = [0] * n_groups                           # pages held now (entries of the table that are >= 0)
 
 
 class CacheManager:
@@ -240,7 +241,7 @@ class CacheManager:
         return slot
 
     def _held(self, state: _SlotState, g: int) -> int:
-        return sum(1 for p in state.tables[g] if p >= 0)
+        return state.held[g]
 
     def _owed(self, state: _SlotState, g: int) -> int:
         """Pages promised to the request that it does not hold yet."""
@@ -264,6 +265,7 @@ class CacheManager:
             if needs[g]:
                 before = self._owed(state, g)
                 state.tables[g].extend(grp.pool.take(needs[g]))
+                state.held[g] += needs[g]
                 grp.pool.promised_unheld += self._owed(state, g) - before
         state.length = length
 
@@ -285,6 +287,7 @@ class CacheManager:
                     state.tables[g][logical] = -1
             state.first_page[g] = max(state.first_page[g], dead_below)
             if dead:
+                state.held[g] -= len(dead)
                 grp.pool.give_back(dead)
                 # a promise covers the pages held at one time: a page given back is owed again
                 grp.pool.promised_unheld += self._owed(state, g) - before
@@ -338,6 +341,9 @@ class CacheManager:
                 raise AssertionError(f"group {g}: pages both held and free: {sorted(set(free) & set(seen))}")
             if len(free) + len(seen) != grp.pool.n_pages:
                 raise AssertionError(f"group {g}: {grp.pool.n_pages - len(free) - len(seen)} pages lost")
+            for slot, state in self._slots.items():
+                if state.held[g] != sum(1 for p in state.tables[g] if p >= 0):
+                    raise AssertionError(f"group {g}: slot {slot} counts {state.held[g]} pages held, its table says otherwise")
             owed = sum(self._owed(s, g) for s in self._slots.values())
             if owed != grp.pool.promised_unheld:
                 raise AssertionError(f"group {g}: promises {grp.pool.promised_unheld} != owed {owed}")

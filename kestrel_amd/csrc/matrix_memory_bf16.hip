@@ -111,8 +111,9 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
                     STs[j * LQ + dd] = (bf16_t)S[jb][db][i];
                 }
         // queries and keys as they are (rows behind the row's last token: zeros), keys and values transposed
+        // (neighbouring lanes take neighbouring tokens: the transposed tiles are then written along their rows)
         for (int e = tid; e < MC_CHUNK * (D / 8); e += MC_THREADS) {
-            const int t = e / (D / 8), piece = e % (D / 8);
+            const int t = e % MC_CHUNK, piece = e / MC_CHUNK;
             mc_bf16x8 qv, kv;
 #pragma unroll
             for (int u = 0; u < 8; ++u) { qv[u] = (bf16_t)0.f; kv[u] = (bf16_t)0.f; }
@@ -127,7 +128,7 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
             for (int u = 0; u < 8; ++u) KTs[(piece * 8 + u) * LC + t] = kv[u];
         }
         for (int e = tid; e < MC_CHUNK * (DV / 8); e += MC_THREADS) {
-            const int t = e / (DV / 8), piece = e % (DV / 8);
+            const int t = e % MC_CHUNK, piece = e / MC_CHUNK;
             mc_bf16x8 vv;
 #pragma unroll
             for (int u = 0; u < 8; ++u) vv[u] = (bf16_t)0.f;

@@ -55,7 +55,7 @@ KA_API int ka_rmsnorm(const float* x, const int* rows, const float* gain, float 
 }
 
 // ----------------------------------------------------------------------------
-// Queries, keys and values of a step made ready for attention, a workgroup per token.
+// Queries, keys and values of a step made ready for attention, a workgroup per token, a wave per head in turns.
 // Row of `qkv`: [H hd queries | G hd keys | G hdv values]. In this order:
 //  * norm (norm_mode 1: every query and key head divided by its root mean square, gains [hd] shared by the
 //    heads; 2: all queries of the token by the root mean square over the whole H hd, likewise all keys, gains
@@ -65,8 +65,8 @@ KA_API int ka_rmsnorm(const float* x, const int* rows, const float* gain, float 
 //  * queries times 1 + q_coef * ln(floor((place + 1) / q_every) + 1) (q_every 0: no such factor);
 //  * values: blend 1 copies them to `v_other` (the values of this layer for later ones), blend 2 replaces them by
 //    (1 - lambda) v + lambda v_other with the fp32 scalar at `lambda`;
-//  * queries go back in place, keys in place and into the paged cache [pages, G, page_size, hd], values into
-//    [pages, G, hdv, page_size] (slots[t] = page * page_size + offset, negative or no slots: nothing is cached).
+//  * queries go back in place; keys go into the paged cache [pages, G, page_size, hd] (the row keeps them as projected),
+//    values into [pages, G, hdv, page_size] (slots[t] = page * page_size + offset, negative or no slots: nothing is cached).
 // ----------------------------------------------------------------------------
 struct PrepareArgs {
     void* qkv;
@@ -94,85 +94,83 @@ template <typename T>
 __global__ void __launch_bounds__(MP_THREADS) qkv_prepare_kernel(PrepareArgs a) {
     extern __shared__ float sm[];
     const int t = blockIdx.x, tid = threadIdx.x;
-    const int heads = a.H + a.G, QK = heads * a.hd, half = a.rot / 2;
-    float* xs = sm;                    // the token's queries and keys as read
-    float* ss = xs + QK;               // sum of squares per head
-    float* cs = ss + heads;            // cosines, then sines, of the token's angles
+    const int wave = tid / KA_WAVE, lane = tid % KA_WAVE;
+    const int heads = a.H + a.G, half = a.rot / 2, hd = a.hd;
+    float* cs = sm;                    // cosines, then sines, of the token's angles
     float* sn = cs + half;
+    float* ss = sn + half;             // sum of squares per head
     T* row = reinterpret_cast<T*>(a.qkv) + (size_t)t * a.row_stride;
     const int pos = a.positions ? a.positions[t] : 0;
-    for (int e = tid; e < QK; e += MP_THREADS) xs[e] = ka_to_float(row[e]);
     if (a.freqs)
         for (int i = tid; i < half; i += MP_THREADS) sincosf((float)pos * a.freqs[i], &sn[i], &cs[i]);
-    __syncthreads();
+    // a wave per head, in turns
     if (a.norm_mode) {
-        const int wave = tid / KA_WAVE, lane = tid % KA_WAVE;
         for (int h = wave; h < heads; h += MP_WAVES) {
+            const T* hp = row + (size_t)h * hd;
             float s = 0.f;
-            for (int c = lane; c < a.hd; c += KA_WAVE) s += xs[h * a.hd + c] * xs[h * a.hd + c];
+            for (int c = lane; c < hd; c += KA_WAVE) {
+                const float x = ka_to_float(hp[c]);
+                s += x * x;
+            }
             s = ka_wave_sum(s);
             if (lane == 0) ss[h] = s;
         }
-        __syncthreads();
     }
+    __syncthreads();
     float r_all_q = 1.f, r_all_k = 1.f;
     if (a.norm_mode == 2) {
         float sq = 0.f, sk = 0.f;
         for (int h = 0; h < a.H; ++h) sq += ss[h];
         for (int h = a.H; h < heads; ++h) sk += ss[h];
-        r_all_q = 1.0f / sqrtf(sq / (float)(a.H * a.hd) + a.eps);
-        r_all_k = 1.0f / sqrtf(sk / (float)(a.G * a.hd) + a.eps);
+        r_all_q = 1.0f / sqrtf(sq / (float)(a.H * hd) + a.eps);
+        r_all_k = 1.0f / sqrtf(sk / (float)(a.G * hd) + a.eps);
     }
     const float q_factor = a.q_every > 0 ? 1.0f + a.q_coef * logf((float)((pos + 1) / a.q_every + 1)) : 1.0f;
     const long slot = a.slots ? a.slots[t] : -1;
     const long page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
     T* k_cache = reinterpret_cast<T*>(a.k_cache);
     T* v_cache = reinterpret_cast<T*>(a.v_cache);
-    for (int e = tid; e < QK; e += MP_THREADS) {
-        const int h = e / a.hd, c = e % a.hd;
+    for (int h = wave; h < heads; h += MP_WAVES) {
         const bool is_q = h < a.H;
+        if (!is_q && slot < 0) continue;            // (a key that is cached nowhere: nobody reads it)
+        T* hp = row + (size_t)h * hd;
+        // where the head's results go: queries back in place, keys into the cache
+        T* dst = is_q ? hp : k_cache + (((size_t)page * a.G + (h - a.H)) * a.page_size + off) * hd;
         float r = 1.f;
-        const float* gain = is_q ? a.q_gain : a.k_gain;
-        int gain_at = 0;                // index of channel 0 of this head in the gains
-        if (a.norm_mode == 1) r = 1.0f / sqrtf(ss[h] / (float)a.hd + a.eps);
-        else if (a.norm_mode == 2) {
+        const float* gain = nullptr;
+        if (a.norm_mode == 1) {
+            r = 1.0f / sqrtf(ss[h] / (float)hd + a.eps);
+            gain = is_q ? a.q_gain : a.k_gain;
+        } else if (a.norm_mode == 2) {
             r = is_q ? r_all_q : r_all_k;
-            gain_at = (is_q ? h : h - a.H) * a.hd;
+            gain = is_q ? a.q_gain : a.k_gain;
+            if (gain) gain += (size_t)(is_q ? h : h - a.H) * hd;
         }
-        const float own = xs[e] * r * (gain && a.norm_mode ? gain[gain_at + c] : 1.f);
-        float y = own;
-        if (a.freqs && c < a.rot) {
-            int i, partner;
-            bool first;
-            if (a.interleaved) { i = c >> 1; first = (c & 1) == 0; partner = c ^ 1; }
-            else { first = c < half; i = first ? c : c - half; partner = first ? c + half : c - half; }
-            const float other = xs[h * a.hd + partner] * r * (gain && a.norm_mode ? gain[gain_at + partner] : 1.f);
-            y = first ? own * cs[i] - other * sn[i] : own * cs[i] + other * sn[i];
+        const float after = is_q ? q_factor : 1.f;
+        // a rotated pair is one lane's: both of its channels are read before either is written
+        if (a.freqs) {
+            for (int i = lane; i < half; i += KA_WAVE) {
+                const int ia = a.interleaved ? 2 * i : i, ib = a.interleaved ? 2 * i + 1 : i + half;
+                const float u = ka_to_float(hp[ia]) * r * (gain ? gain[ia] : 1.f);
+                const float v = ka_to_float(hp[ib]) * r * (gain ? gain[ib] : 1.f);
+                dst[ia] = ka_from_float<T>((u * cs[i] - v * sn[i]) * after);
+                dst[ib] = ka_from_float<T>((v * cs[i] + u * sn[i]) * after);
+            }
         }
-        if (is_q) {
-            row[e] = ka_from_float<T>(y * q_factor);
-        } else {
-            const T stored = ka_from_float<T>(y);
-            row[e] = stored;
-            if (slot >= 0) k_cache[(((size_t)page * a.G + (h - a.H)) * a.page_size + off) * a.hd + c] = stored;
-        }
+        for (int c = a.rot + lane; c < hd; c += KA_WAVE)
+            dst[c] = ka_from_float<T>(ka_to_float(hp[c]) * r * (gain ? gain[c] : 1.f) * after);
     }
-    T* vrow = row + QK;
-    const int VN = a.G * a.hdv;
+    T* vrow = row + (size_t)heads * hd;
     const float lam = a.blend == 2 ? *a.lambda : 0.f;
     T* other = a.blend ? reinterpret_cast<T*>(a.v_other) + (size_t)t * a.v_other_stride : nullptr;
-    for (int e = tid; e < VN; e += MP_THREADS) {
-        T v = vrow[e];
-        if (a.blend == 1) other[e] = v;
-        else if (a.blend == 2) {
-            v = ka_from_float<T>((1.0f - lam) * ka_to_float(v) + lam * ka_to_float(other[e]));
-            vrow[e] = v;
+    for (int g = wave; g < a.G; g += MP_WAVES)
+        for (int c = lane; c < a.hdv; c += KA_WAVE) {
+            const int e = g * a.hdv + c;
+            T v = vrow[e];
+            if (a.blend == 1) other[e] = v;
+            else if (a.blend == 2) v = ka_from_float<T>((1.0f - lam) * ka_to_float(v) + lam * ka_to_float(other[e]));
+            if (slot >= 0) v_cache[(((size_t)page * a.G + g) * a.hdv + c) * a.page_size + off] = v;
         }
-        if (slot >= 0) {
-            const int g = e / a.hdv, c = e % a.hdv;
-            v_cache[(((size_t)page * a.G + g) * a.hdv + c) * a.page_size + off] = v;
-        }
-    }
 }
 
 KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* positions, const int* slots, void* k_cache,
@@ -195,8 +193,8 @@ KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* posi
     KA_CHECK(dtype == KA_F32 || dtype == KA_BF16, "%s: unsupported dtype %d", who, dtype);
     if (n == 0) return 0;
     if (freqs == nullptr) rot = 0;
-    const size_t lds = ((size_t)(H + G) * hd + (H + G) + rot) * sizeof(float);
-    KA_CHECK(lds <= 64 * 1024, "%s: a token's queries and keys (%d values) do not fit in LDS", who, (H + G) * hd);
+    const size_t lds = ((size_t)(H + G) + rot) * sizeof(float);
+    KA_CHECK(lds <= 64 * 1024, "%s: %d heads and %d rotated channels do not fit in LDS", who, H + G, rot);
     PrepareArgs a{qkv, row_stride, positions, slots, k_cache, v_cache, H, G, hd, hdv, page_size, norm_mode, q_gain, k_gain, eps,
                   freqs, rot, interleaved, q_coef, q_every, blend, v_other, v_other_stride, lambda};
     if (dtype == KA_F32) hipLaunchKernelGGL(qkv_prepare_kernel<float>, dim3(n), dim3(MP_THREADS), lds, stream, a);
@@ -224,6 +222,42 @@ KA_API int ka_gate_mul(void* x, long x_stride, const void* gate, long gate_strid
         hipLaunchKernelGGL(gate_mul_kernel<float>, dim3(n), dim3(MP_THREADS), 0, stream, (float*)x, x_stride, (const float*)gate, gate_stride, dim);
     else
         hipLaunchKernelGGL(gate_mul_kernel<bf16_t>, dim3(n), dim3(MP_THREADS), 0, stream, (bf16_t*)x, x_stride, (const bf16_t*)gate, gate_stride, dim);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// The product of a gated pair: out[t, j] = act(x[t, 2j]) * x[t, 2j + 1] for rows whose gate and value sums lie side by
+// side (what a plain linear over paired weight rows leaves): the second half of a gated linear whose first half went
+// through a kernel that has no such epilogue (the vendor library's). Rows of the activation type.
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(MP_THREADS)
+gated_pairs_kernel(const T* __restrict__ x, long x_stride, T* __restrict__ out, long out_stride, int n_out, int act) {
+    const T* xr = x + (size_t)blockIdx.y * x_stride;
+    T* orow = out + (size_t)blockIdx.y * out_stride;
+    typedef T __attribute__((ext_vector_type(2))) pair_t;
+    for (int j = blockIdx.x * MP_THREADS + threadIdx.x; j < n_out; j += gridDim.x * MP_THREADS) {
+        const pair_t p = *reinterpret_cast<const pair_t*>(xr + 2 * (size_t)j);
+        const float g = sizeof(T) == 2 ? ka_activate_fast(act, ka_to_float(p[0])) : ka_activate(act, ka_to_float(p[0]));
+        orow[j] = ka_from_float<T>(g * ka_to_float(p[1]));
+    }
+}
+
+KA_API int ka_gated_pairs(const void* x, long x_stride, void* out, long out_stride, int dtype, int n, int n_out, int act,
+                          hipStream_t stream) {
+    KA_CHECK(n >= 0 && n_out > 0 && x_stride >= 2L * n_out && out_stride >= n_out && x_stride % 2 == 0, "ka_gated_pairs: bad sizes");
+    KA_CHECK(dtype == KA_F32 || dtype == KA_BF16, "ka_gated_pairs: unsupported dtype %d", dtype);
+    KA_CHECK(ka_act_known(act) && !ka_act_gated(act), "ka_gated_pairs: unknown activation %d", act);
+    KA_CHECK(n <= 65535, "ka_gated_pairs: too many rows %d", n);
+    KA_CHECK((uintptr_t)x % (dtype == KA_F32 ? 8 : 4) == 0, "ka_gated_pairs: pairs must be aligned");
+    if (n == 0) return 0;
+    const int blocks = ka_cdiv(n_out, MP_THREADS * 4) < 1 ? 1 : ka_cdiv(n_out, MP_THREADS * 4);
+    const dim3 grid(blocks, n);
+    if (dtype == KA_F32)
+        hipLaunchKernelGGL(gated_pairs_kernel<float>, grid, dim3(MP_THREADS), 0, stream, (const float*)x, x_stride, (float*)out, out_stride, n_out, act);
+    else
+        hipLaunchKernelGGL(gated_pairs_kernel<bf16_t>, grid, dim3(MP_THREADS), 0, stream, (const bf16_t*)x, x_stride, (bf16_t*)out, out_stride, n_out, act);
     KA_LAUNCH_CHECK();
     return 0;
 }

@@ -36,6 +36,7 @@ _SIGNATURES = {
     "ka_qkv_prepare": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                        _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_float, _c_int,
                        _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p],
+    "ka_gated_pairs": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_gate_mul": [_c_void_p, _c_long, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_void_p],
     "ka_branches_sum": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_void_p, _c_float, _c_float, _c_int, _c_int,
                         _c_void_p],
@@ -358,7 +359,8 @@ def qkv_prepare(qkv: torch.Tensor, positions: Optional[torch.Tensor], slots: Opt
     then the rotation of the first ``2 len(freqs)`` channels of every head by ``place * freqs`` (fp32 ``freqs``; ``pairing`` as
     in ``rope_cache``), then queries times ``1 + coef * ln(floor((place + 1) / every) + 1)`` for ``q_growth = (coef, every)``;
     values copied to ``v_other`` (``blend`` ``"source"``) or replaced by ``(1 - w) v + w v_other`` (``"blend"``, ``w`` the fp32
-    scalar tensor ``blend_weight``); queries and keys back in place, keys and values into the paged cache at ``slots``."""
+    scalar tensor ``blend_weight``); queries back in place, keys and values into the paged cache at ``slots`` (the rows keep
+    keys and values as they were projected)."""
     _need(pairing in ROTARY_PAIRINGS, f"qkv_prepare: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     _need(norm_scope in QK_NORM_SCOPES and blend in VALUE_BLENDS, "qkv_prepare: unknown norm scope or blend")
     _dev(qkv, positions, slots, k_cache, v_cache, q_gain, k_gain, freqs, v_other, blend_weight)
@@ -390,6 +392,17 @@ def qkv_prepare(qkv: torch.Tensor, positions: Optional[torch.Tensor], slots: Opt
                                 QK_NORM_SCOPES[norm_scope], _ptr(q_gain), _ptr(k_gain), float(eps), _ptr(freqs), rot,
                                 ROTARY_PAIRINGS[pairing], coef, every, VALUE_BLENDS[blend], _ptr(v_other),
                                 (v_other.stride(0) if n > 1 else n_kv_heads * value_dim) if v_other is not None else 0, _ptr(blend_weight), stream_ptr()))
+
+
+def gated_pairs(x: torch.Tensor, out: torch.Tensor, act: int) -> None:
+    """``out[:, j] = act(x[:, 2 j]) * x[:, 2 j + 1]``: the product of the pairs that a plain linear over paired weight rows
+    (``ops.linear.pair_rows``) leaves side by side; ``act`` an activation's code without the gated flag."""
+    _dev(x, out)
+    n, n_out = out.shape
+    _need(x.dim() == 2 and tuple(x.shape) == (n, 2 * n_out) and x.dtype == out.dtype and x.stride(1) == 1 and out.stride(1) == 1,
+          "gated_pairs: x must be [n, 2 m] and out [n, m] of one type")
+    _check(lib().ka_gated_pairs(x.data_ptr(), x.stride(0) if n > 1 else 2 * n_out, out.data_ptr(), out.stride(0) if n > 1 else n_out,
+                                code_of(x.dtype), n, n_out, int(act), stream_ptr()))
 
 
 def gate_mul(x: torch.Tensor, gate: torch.Tensor) -> None:

@@ -90,9 +90,21 @@ class GatedFeedForward(FeedForward):
     def output_projection(self):
         return self.down_weight, self.down_bias
 
+    # Rows from which the gated linear is run as a plain linear over all paired rows (the vendor library's kernels, which
+    # have no epilogue for the product of a pair) followed by a pass that takes the products: at 2,048 rows of width 2,048
+    # and 5,632 pairs 100 us against the 169 of this package's tiled kernel with the product in its epilogue.
+    PAIRS_APART_FROM_ROWS = 256
+
     def forward(self, h, batch, residual) -> None:
-        hidden = batch.workspace.get("ff.hidden", (h.shape[0], self.spec.hidden_dim), self.dtype)
-        linear_gated(h, self.pairs, self.pair_bias, hidden, self.act)
+        n = h.shape[0]
+        hidden = batch.workspace.get("ff.hidden", (n, self.spec.hidden_dim), self.dtype)
+        if self.dtype == torch.bfloat16 and n >= self.PAIRS_APART_FROM_ROWS:
+            from ..ops import core
+            sums = batch.workspace.get("ff.pair_sums", (n, 2 * self.spec.hidden_dim), self.dtype)
+            linear(h, self.pairs, self.pair_bias, sums)
+            core.gated_pairs(sums, hidden, self.act)
+        else:
+            linear_gated(h, self.pairs, self.pair_bias, hidden, self.act)
         linear(hidden, self.down_weight, self.down_bias, residual, accumulate=True)
 
 
