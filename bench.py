@@ -287,7 +287,7 @@ def run_compare_bogivik(args, dtype, device) -> dict:
     size_bytes = 2 if dtype == torch.bfloat16 else 4
     context, tokens = args.context, args.prefill_tokens
     positions = max(context + args.steps + args.warmup + 16, tokens)
-    labels = [label for label in args.compare_sizes.split(",") if label in BOGIVIK_SIZES] or list(BOGIVIK_SIZES)
+    labels = (args.compare_sizes or ",".join(BOGIVIK_SIZES)).split(",")
     out = {}
     for label in labels:
         out[label] = {}
@@ -614,8 +614,9 @@ def main() -> int:
     parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48", "compare-vimesun", "compare-bogivik"],
                         help="decode: the benchmark's decode step (default); waves256 and mixed48 run requests through "
                              "InferenceEngine; compare-vimesun and compare-bogivik measure that design beside the Moondream decoder at equal sizes")
-    parser.add_argument("--compare-sizes", default="w2048,w2048-window,w4096-gqa,w2560-v",
-                        help="with --workload compare-vimesun: which of the sizes, with commas between them")
+    parser.add_argument("--compare-sizes", default=None,
+                        help="with --workload compare-vimesun or compare-bogivik: which of its sizes, with commas between them "
+                             "(default: all of them)")
     parser.add_argument("--compare-model", default="both", choices=["both", "vimesun", "bogivik", "moondream2"],
                         help="with --workload compare-*: one of the two designs only (for profiling)")
     parser.add_argument("--compare-batches", default="1,8,64", help="with --workload compare-bogivik: batch sizes of the decode steps")
@@ -646,6 +647,7 @@ def main() -> int:
     if args.layers is None:
         args.layers = sizes["n_layers"]
     if args.workload == "compare-vimesun":
+        args.compare_sizes = args.compare_sizes or ",".join(COMPARE_SIZES)
         print(json.dumps(run_compare(args, dtype, device)))
         return 0
     if args.workload == "compare-bogivik":

@@ -12,7 +12,15 @@
 // Gates, maxima, weights, sums, the state and the norm of the read-out are fp32; P, the weighted values and a copy of
 // S_0 enter the products as bf16 (as the weights of attention do).
 //
-// A workgroup of four waves per (head, row of the batch) walks over the row's chunks. S^T lives in the accumulators of
+// Two ways of running it. In turn: a workgroup of four waves per (head, row of the batch) walks over the row's chunks
+// (MC_SEQ). In three passes, for rows of many chunks: every chunk's state as if it started from nothing, all chunks at
+// once (MC_LOCAL: e^(a_s - max a) weights, its own maximum m_loc = F_L + max a); a scan over a row's chunks that turns
+// those into the state every chunk starts from, m_end = max(F_L + m_start, m_loc),
+// S_end = e^(F_L + m_start - m_end) S_start + e^(m_loc - m_end) S_loc, element by element in fp32 (it also advances the
+// request's state); and every chunk's read-out from its start state, all chunks at once (MC_READ). The passes meet in a
+// buffer of the caller's, per chunk and head S [d, dv], n [d], m and F_L.
+//
+// In turn, a workgroup of four waves per (head, row of the batch) walks over the row's chunks. S^T lives in the accumulators of
 // the state product for the whole walk: wave w owns the value channels [w dv / 4, (w + 1) dv / 4). Operands are staged in
 // LDS in the layouts that v_mfma_f32_32x32x16_bf16 reads with one 16-byte load a lane: a row operand as [row][k], a
 // column operand as [column][k].
@@ -24,6 +32,8 @@ typedef __attribute__((ext_vector_type(16))) float mc_floatx16;
 constexpr int MC_CHUNK = 64;
 constexpr int MC_THREADS = 256;
 constexpr int MC_PAD = 8;                   // elements a row of an LDS tile is longer than its data: spreads rows over banks
+constexpr int MC_SEQ = 0, MC_LOCAL = 1, MC_READ = 2;
+constexpr int MC_SCAN_CHUNKS = 1024;        // most chunks of one row that the scan keeps the weights of in LDS
 
 struct ChunkArgs {
     const bf16_t* q; const bf16_t* k; const bf16_t* v; const bf16_t* gate;
@@ -37,7 +47,25 @@ struct ChunkArgs {
     long out_stride;
     int heads;
     float q_scale, cap, eps;
+    float* chunks;                 // the passes' buffer: fp32 [chunks, heads, d dv + d + 2]
+    int n_rows;
 };
+
+// The row and the first token of chunk `g` of the batch (chunks numbered row by row); false: behind the last chunk.
+__device__ __forceinline__ bool mc_find_chunk(const int* cu_q, int n_rows, int g, int& r, int& t0, int& t1, int& c0) {
+    int base = 0;
+    for (r = 0; r < n_rows; ++r) {
+        t0 = cu_q[r];
+        t1 = cu_q[r + 1];
+        const int nc = (t1 - t0 + MC_CHUNK - 1) / MC_CHUNK;
+        if (g < base + nc) {
+            c0 = t0 + (g - base) * MC_CHUNK;
+            return true;
+        }
+        base += nc;
+    }
+    return false;
+}
 
 __device__ __forceinline__ float mc_running_max(float x, int lane) {
     for (int off = 1; off < KA_WAVE; off <<= 1) {
@@ -47,8 +75,8 @@ __device__ __forceinline__ float mc_running_max(float x, int lane) {
     return x;
 }
 
-// ND: d = 32 ND; NJ: dv = 128 NJ.
-template <int ND, int NJ>
+// ND: d = 32 ND; NJ: dv = 128 NJ. MODE: MC_SEQ (grid (heads, rows)), MC_LOCAL or MC_READ (grid (heads, chunks)).
+template <int ND, int NJ, int MODE>
 __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkArgs a) {
     constexpr int D = 32 * ND, DV = 128 * NJ, WJ = 32 * NJ;       // WJ: value channels a wave owns
     constexpr int LQ = D + MC_PAD, LC = MC_CHUNK + MC_PAD;
@@ -68,20 +96,31 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
     float* sq = rowsum + 2 * MC_CHUNK;                            // [4][64]: sums of squares of the read-out by wave
     float* nvec = sq + 4 * MC_CHUNK;                              // [D]: n
     float* nnew = nvec + D;                                       // [D]
-    float* scal = nnew + D;                                       // [2]: m_0 of the next chunk, c_L
+    float* scal = nnew + D;                                       // [3]: m_0 of the next chunk, c_L, F_L
 
-    const int head = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+    const int head = blockIdx.x, tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid / KA_WAVE), lane = tid % KA_WAVE;
     const int col = lane % 32, half = lane / 32;
-    const int t0 = a.cu_q[r], t1 = a.cu_q[r + 1];
+    int r = blockIdx.y, t0, t1, first = 0;
+    if constexpr (MODE == MC_SEQ) {
+        t0 = a.cu_q[r];
+        t1 = a.cu_q[r + 1];
+        first = t0;
+    } else {
+        if (!mc_find_chunk(a.cu_q, a.n_rows, blockIdx.y, r, t0, t1, first)) return;
+        t1 = min(t1, first + MC_CHUNK);                 // (this workgroup's chunk alone)
+    }
     if (t0 >= t1) return;
     const int slot = a.row_slot[r];
     if (slot < 0) {
-        for (int t = t0; t < t1; ++t)
-            for (int j = tid; j < DV; j += MC_THREADS) a.out[(size_t)t * a.out_stride + head * DV + j] = (bf16_t)0.f;
+        if constexpr (MODE != MC_LOCAL)
+            for (int t = first; t < t1; ++t)
+                for (int j = tid; j < DV; j += MC_THREADS) a.out[(size_t)t * a.out_stride + head * DV + j] = (bf16_t)0.f;
         return;
     }
-    float* st = a.state + ((size_t)slot * a.heads + head) * (D * DV + D + 1);
+    // where the state comes from and goes to: the request's row (in turn), the chunk's record of the passes' buffer
+    float* st = MODE == MC_SEQ ? a.state + ((size_t)slot * a.heads + head) * (D * DV + D + 1)
+                               : a.chunks + ((size_t)blockIdx.y * a.heads + head) * (D * DV + D + 2);
     // S^T in accumulators: tile (jb, db), register i of a lane: value channel wave WJ + jb 32 + (i / 4) 8 + half 4 + i % 4,
     // key channel db 32 + col
     mc_floatx16 S[NJ][ND];
@@ -92,24 +131,28 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int j = wave * WJ + jb * 32 + (i / 4) * 8 + half * 4 + i % 4, dd = db * 32 + col;
-                S[jb][db][i] = st[(size_t)dd * DV + j];
+                S[jb][db][i] = MODE == MC_SEQ ? st[(size_t)dd * DV + j] : 0.f;
             }
-    for (int e = tid; e < D; e += MC_THREADS) nvec[e] = st[D * DV + e];
-    float m0 = st[D * DV + D];
+    for (int e = tid; e < D; e += MC_THREADS) nvec[e] = MODE == MC_LOCAL ? 0.f : st[D * DV + e];
+    float m0 = MODE == MC_LOCAL ? -INFINITY : st[D * DV + D];      // (a chunk as if it started from nothing)
 
-    for (int c0 = t0; c0 < t1; c0 += MC_CHUNK) {
+    for (int c0 = first; c0 < t1; c0 += MC_CHUNK) {
         const int valid = min(MC_CHUNK, t1 - c0);
         __syncthreads();                   // (the chunk before is done with every tile)
         // the state the chunk starts from, as a column operand
+        if constexpr (MODE == MC_SEQ) {
 #pragma unroll
-        for (int jb = 0; jb < NJ; ++jb)
+            for (int jb = 0; jb < NJ; ++jb)
 #pragma unroll
-            for (int db = 0; db < ND; ++db)
+                for (int db = 0; db < ND; ++db)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int j = wave * WJ + jb * 32 + (i / 4) * 8 + half * 4 + i % 4, dd = db * 32 + col;
-                    STs[j * LQ + dd] = (bf16_t)S[jb][db][i];
-                }
+                    for (int i = 0; i < 16; ++i) {
+                        const int j = wave * WJ + jb * 32 + (i / 4) * 8 + half * 4 + i % 4, dd = db * 32 + col;
+                        STs[j * LQ + dd] = (bf16_t)S[jb][db][i];
+                    }
+        } else if constexpr (MODE == MC_READ) {
+            for (int e = tid; e < D * DV; e += MC_THREADS) STs[(e % DV) * LQ + e / DV] = (bf16_t)st[e];
+        }
         // queries and keys as they are (rows behind the row's last token: zeros), keys and values transposed
         // (neighbouring lanes take neighbouring tokens: the transposed tiles are then written along their rows)
         for (int e = tid; e < MC_CHUNK * (D / 8); e += MC_THREADS) {
@@ -156,9 +199,11 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
             if (lane == 0) {
                 scal[0] = ka_lane_value(F + top, KA_WAVE - 1);
                 scal[1] = expf(m0 + b_last);
+                scal[2] = ka_lane_value(F, KA_WAVE - 1);
             }
         }
         __syncthreads();
+        if constexpr (MODE != MC_LOCAL) {
         // n_0 . q_t, a token a thread
         if (tid < MC_CHUNK) {
             float acc = 0.f;
@@ -254,6 +299,8 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
                     }
                 }
             }
+        }   // (MODE != MC_LOCAL)
+        if constexpr (MODE == MC_READ) return;
         // the state after the chunk: S^T <- c_L S^T + (diag(u) V)^T K, n <- c_L n + K^T u
         const float c_last = scal[1];
         if (tid < D) {
@@ -296,14 +343,70 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
                 st[(size_t)dd * DV + j] = S[jb][db][i];
             }
     for (int e = tid; e < D; e += MC_THREADS) st[D * DV + e] = nvec[e];
-    if (tid == 0) st[D * DV + D] = m0;
+    if (tid == 0) {
+        st[D * DV + D] = m0;
+        if constexpr (MODE == MC_LOCAL) st[D * DV + D + 1] = scal[2];
+    }
+}
+
+// The scan of the three passes: a workgroup per (head, row). Thread 0 walks over the row's chunks and leaves, per chunk,
+// the two weights of its step and the maximum it starts from; every thread then carries its share of S and n through the
+// chunks, writing into each chunk's record the state it starts from, and the request's state at the end.
+__global__ void __launch_bounds__(MC_THREADS) matrix_memory_scan_kernel(ChunkArgs a, int D, int DV) {
+    __shared__ float w_old[MC_SCAN_CHUNKS], w_new[MC_SCAN_CHUNKS];
+    const int head = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
+    const int t0 = a.cu_q[r], t1 = a.cu_q[r + 1];
+    if (t0 >= t1) return;
+    const int slot = a.row_slot[r];
+    if (slot < 0) return;
+    int base = 0;
+    for (int q = 0; q < r; ++q) base += (a.cu_q[q + 1] - a.cu_q[q] + MC_CHUNK - 1) / MC_CHUNK;
+    const int nc = (t1 - t0 + MC_CHUNK - 1) / MC_CHUNK;
+    const int per = D * DV + D;
+    float* st = a.state + ((size_t)slot * a.heads + head) * (per + 1);
+    float* rec = a.chunks + ((size_t)base * a.heads + head) * (per + 2);
+    const size_t step = (size_t)a.heads * (per + 2);
+    if (tid == 0) {
+        float m = st[per];
+        for (int c = 0; c < nc; ++c) {
+            float* at = rec + c * step;
+            const float m_loc = at[per], f_all = at[per + 1];
+            const float m_end = fmaxf(f_all + m, m_loc);
+            w_old[c] = expf(f_all + m - m_end);
+            w_new[c] = expf(m_loc - m_end);
+            at[per] = m;                    // the maximum the chunk starts from
+            m = m_end;
+        }
+        st[per] = m;
+    }
+    __syncthreads();
+    for (int e = tid; e < per; e += MC_THREADS) {
+        float cur = st[e];
+        int c = 0;
+        for (; c + 3 < nc; c += 4) {        // (four records in flight)
+            float x[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) x[u] = rec[(c + u) * step + e];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                rec[(c + u) * step + e] = cur;
+                cur = w_old[c + u] * cur + w_new[c + u] * x[u];
+            }
+        }
+        for (; c < nc; ++c) {
+            const float x = rec[c * step + e];
+            rec[c * step + e] = cur;
+            cur = w_old[c] * cur + w_new[c] * x;
+        }
+        st[e] = cur;
+    }
 }
 
 template <int ND, int NJ>
 static size_t mc_lds_bytes() {
     constexpr int D = 32 * ND, DV = 128 * NJ, LQ = D + MC_PAD, LC = MC_CHUNK + MC_PAD;
     return sizeof(bf16_t) * ((size_t)2 * MC_CHUNK * LQ + (size_t)D * LC + (size_t)DV * LC + (size_t)MC_CHUNK * LC + (size_t)DV * LQ)
-        + sizeof(float) * (5 * MC_CHUNK + 2 * MC_CHUNK + 4 * MC_CHUNK + 2 * D + 2);
+        + sizeof(float) * (5 * MC_CHUNK + 2 * MC_CHUNK + 4 * MC_CHUNK + 2 * D + 4);
 }
 
 // Whether the kernel covers heads of these sizes: keys of 32, 64 or 128 channels, values of 128 or 256 (128 x 256: its
@@ -312,10 +415,17 @@ KA_API int ka_matrix_memory_chunks_supported(int d, int dv) {
     return (d == 32 || d == 64 || d == 128) && (dv == 128 || dv == 256) && !(d == 128 && dv == 256) ? 1 : 0;
 }
 
+// Floats of the passes' buffer for a step of `n` tokens in `n_rows` rows (every row may end in a part of a chunk).
+KA_API long ka_matrix_memory_chunks_scratch(int n, int n_rows, int heads, int d, int dv) {
+    return (long)(n / MC_CHUNK + n_rows) * heads * ((long)d * dv + d + 2);
+}
+
+// chunks != nullptr (of at least ka_matrix_memory_chunks_scratch floats; n = the step's tokens): the three passes;
+// nullptr: every row's chunks in turn.
 KA_API int ka_matrix_memory_chunks_bf16(const void* q, const void* k, const void* v, const void* gate, long stride,
                                         const float* pre, float* state, const int* cu_q, const int* row_slot,
                                         const float* gain, void* out, long out_stride, int n_rows, int heads, int d, int dv,
-                                        float q_scale, float cap, float eps, hipStream_t stream) {
+                                        float q_scale, float cap, float eps, float* chunks, int n, hipStream_t stream) {
     const char* who = "ka_matrix_memory_chunks_bf16";
     KA_CHECK(n_rows >= 0 && heads > 0 && ka_matrix_memory_chunks_supported(d, dv), "%s: heads of %d x %d not covered", who, d, dv);
     KA_CHECK(cap > 0.f && eps >= 0.f, "%s: the gates' cap must be positive", who);
@@ -323,21 +433,35 @@ KA_API int ka_matrix_memory_chunks_bf16(const void* q, const void* k, const void
     KA_CHECK((uintptr_t)q % 16 == 0 && (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0 && stride % 8 == 0,
              "%s: operands must be 16-byte aligned", who);
     if (n_rows == 0) return 0;
+    const int n_chunks = n / MC_CHUNK + n_rows;
+    // (a row of more chunks than the scan keeps weights for, or more chunks than a grid takes: in turn)
+    if (chunks != nullptr && (n / MC_CHUNK + 1 > MC_SCAN_CHUNKS || n_chunks > 65535)) chunks = nullptr;
     ChunkArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)gate, stride, pre, state, cu_q, row_slot,
-                gain, (bf16_t*)out, out_stride, heads, q_scale, cap, eps};
-    const dim3 grid(heads, n_rows), block(MC_THREADS);
-#define MC_LAUNCH(ND, NJ)                                                                                                   \
-    if (d == 32 * ND && dv == 128 * NJ) {                                                                                   \
+                gain, (bf16_t*)out, out_stride, heads, q_scale, cap, eps, chunks, n_rows};
+    const dim3 block(MC_THREADS);
+#define MC_LAUNCH_MODE(ND, NJ, MODE, GRID)                                                                                  \
+    do {                                                                                                                    \
         static bool sized = false;                                                                                          \
         if (!sized) {                                                                                                       \
-            (void)hipFuncSetAttribute((const void*)matrix_memory_chunk_kernel<ND, NJ>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            (void)hipFuncSetAttribute((const void*)matrix_memory_chunk_kernel<ND, NJ, MODE>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
             sized = true;                                                                                                   \
         }                                                                                                                   \
         const size_t lds = mc_lds_bytes<ND, NJ>();                                                                          \
-        hipLaunchKernelGGL((matrix_memory_chunk_kernel<ND, NJ>), grid, block, lds, stream, a);                              \
+        hipLaunchKernelGGL((matrix_memory_chunk_kernel<ND, NJ, MODE>), GRID, block, lds, stream, a);                        \
+    } while (0)
+#define MC_LAUNCH(ND, NJ)                                                                                                   \
+    if (d == 32 * ND && dv == 128 * NJ) {                                                                                   \
+        if (chunks == nullptr) {                                                                                            \
+            MC_LAUNCH_MODE(ND, NJ, MC_SEQ, dim3(heads, n_rows));                                                            \
+        } else {                                                                                                            \
+            MC_LAUNCH_MODE(ND, NJ, MC_LOCAL, dim3(heads, n_chunks));                                                        \
+            hipLaunchKernelGGL(matrix_memory_scan_kernel, dim3(heads, n_rows), block, 0, stream, a, d, dv);                 \
+            MC_LAUNCH_MODE(ND, NJ, MC_READ, dim3(heads, n_chunks));                                                         \
+        }                                                                                                                   \
     }
     MC_LAUNCH(1, 1) MC_LAUNCH(2, 1) MC_LAUNCH(4, 1) MC_LAUNCH(1, 2) MC_LAUNCH(2, 2)
 #undef MC_LAUNCH
+#undef MC_LAUNCH_MODE
     KA_LAUNCH_CHECK();
     return 0;
 }

@@ -430,7 +430,8 @@ def branches_sum(x: torch.Tensor, a: torch.Tensor, gain_a: Optional[torch.Tensor
 
 def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: torch.Tensor, cu_q: torch.Tensor,
                   row_slot: torch.Tensor, gain: Optional[torch.Tensor], out: torch.Tensor, n_heads: int, head_dim: int,
-                  value_dim: int, q_scale: float, cap: float, eps: float, single_tokens: bool, chunks: bool = False) -> None:
+                  value_dim: int, q_scale: float, cap: float, eps: float, single_tokens: bool, chunks: bool = False,
+                  scratch: Optional[torch.Tensor] = None) -> None:
     """The gated matrix memory over the packed tokens of a step. ``projected`` ``[n, *]`` holds queries, keys, values and
     (optionally) the output gate's pre-activations at the column ``offsets = (q, k, v, gate or None)``; ``pre`` fp32
     ``[n, 2 heads]`` the pre-activations of the input gates, then of the forget gates; ``state`` fp32
@@ -438,7 +439,8 @@ def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: to
     place for row ``r`` at ``row_slot[r]`` over its tokens ``cu_q[r] .. cu_q[r + 1]`` (a negative slot: zeros are written,
     no state is touched). ``out`` ``[n, heads * hdv]``: every head's read-out divided by its root mean square, times ``gain``
     (fp32 ``[heads * hdv]``), times the sigmoid of the gate. ``chunks``: bf16 prompt portions go to the matrix-core kernel that
-    unrolls the recurrence over chunks of 64 tokens, where it covers the sizes (``ops.fast.matrix_memory_chunks_bf16``)."""
+    unrolls the recurrence over chunks of 64 tokens, where it covers the sizes (``ops.fast.matrix_memory_chunks_bf16``; with
+    ``scratch`` of ``ops.fast.matrix_memory_chunks_scratch`` fp32 numbers all chunks of a row at once)."""
     _dev(projected, pre, state, cu_q, row_slot, gain, out)
     n = projected.shape[0]
     n_rows = row_slot.numel()
@@ -458,7 +460,7 @@ def matrix_memory(projected: torch.Tensor, offsets, pre: torch.Tensor, state: to
     if chunks and projected.dtype == torch.bfloat16 and not single_tokens:
         from . import fast
         if fast.matrix_memory_chunks_bf16(projected, offsets, pre, state, cu_q, row_slot, gain, out, n_heads, head_dim, value_dim,
-                                          q_scale, cap, eps):
+                                          q_scale, cap, eps, scratch=scratch):
             return
     size = projected.element_size()
     base = projected.data_ptr()

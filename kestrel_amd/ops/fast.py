@@ -57,7 +57,7 @@ _SIGNATURES = {
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_void_p, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_matrix_memory_chunks_bf16": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                      _c_void_p, _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
-                                     _c_void_p],
+                                     _c_void_p, _c_int, _c_void_p],
     "ka_linear_skinny_norm_store": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p,
                                     _c_int, _c_long, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
 }
@@ -652,11 +652,22 @@ def attention_biased_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
     return True
 
 
+def matrix_memory_chunks_scratch(n: int, n_rows: int, n_heads: int, head_dim: int, value_dim: int) -> int:
+    """fp32 numbers of scratch that ``matrix_memory_chunks_bf16`` needs to run a step of ``n`` tokens in ``n_rows`` rows in
+    three passes (all chunks at once, a scan, all chunks at once); 0: the kernel does not cover the head sizes."""
+    handle = lib()
+    handle.ka_matrix_memory_chunks_scratch.restype = ctypes.c_long
+    if not handle.ka_matrix_memory_chunks_supported(int(head_dim), int(value_dim)):
+        return 0
+    return int(handle.ka_matrix_memory_chunks_scratch(int(n), int(n_rows), int(n_heads), int(head_dim), int(value_dim)))
+
+
 def matrix_memory_chunks_bf16(projected, offsets, pre, state, cu_q, row_slot, gain, out, n_heads, head_dim, value_dim,
-                              q_scale, cap, eps) -> bool:
+                              q_scale, cap, eps, scratch=None) -> bool:
     """``ops.core.matrix_memory`` for prompt portions on the matrix cores: the recurrence unrolled over chunks of 64 tokens
-    (operands as for ``ops.core.matrix_memory``, which has checked them). False: head sizes or alignment not covered,
-    nothing was run."""
+    (operands as for ``ops.core.matrix_memory``, which has checked them). ``scratch`` (fp32, at least
+    ``matrix_memory_chunks_scratch`` numbers): the chunks of every row run at once, in three passes, instead of in turn.
+    False: head sizes or alignment not covered, nothing was run."""
     handle = lib()
     n = projected.shape[0]
     if n == 0:
@@ -668,9 +679,13 @@ def matrix_memory_chunks_bf16(projected, offsets, pre, state, cu_q, row_slot, ga
     stride = projected.stride(0) if n > 1 else projected.shape[1]
     if base % 16 or stride % 8 or any(o % 8 for o in (oq, ok, ov)) or (n_heads * head_dim) % 8:
         return False
+    if scratch is not None:
+        need = matrix_memory_chunks_scratch(n, int(row_slot.numel()), n_heads, head_dim, value_dim)
+        if scratch.dtype != torch.float32 or not scratch.is_contiguous() or scratch.numel() < need:
+            raise KernelError(f"matrix memory: the passes' scratch must be contiguous fp32 of at least {need} numbers")
     _check(handle.ka_matrix_memory_chunks_bf16(base + oq * size, base + ok * size, base + ov * size,
                                                None if og is None else base + og * size, stride, pre.data_ptr(), state.data_ptr(),
                                                cu_q.data_ptr(), row_slot.data_ptr(), _ptr(gain), out.data_ptr(),
                                                out.stride(0) if n > 1 else n_heads * value_dim, int(row_slot.numel()), n_heads,
-                                               head_dim, value_dim, float(q_scale), float(cap), float(eps), stream_ptr()))
+                                               head_dim, value_dim, float(q_scale), float(cap), float(eps), _ptr(scratch), n, stream_ptr()))
     return True

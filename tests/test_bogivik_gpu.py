@@ -431,17 +431,20 @@ def test_gate_and_branches_kernels(dtype):
         assert torch.allclose(out.double().cpu(), base.double() + 2.0 * plain.rms_norm(a.double(), None, 1e-5), rtol=2e-5, atol=2e-5)
 
 
+@pytest.mark.parametrize("passes", [False, True], ids=["in turn", "three passes"])
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
 @pytest.mark.parametrize("heads, d, dv", [(3, 20, 36), (1, 8, 300), (2, 64, 64), (2, 200, 200), (2, 64, 128), (1, 32, 256),
                                           (1, 128, 128), (3, 64, 256)])
-def test_matrix_memory_kernel(heads, d, dv, dtype):
+def test_matrix_memory_kernel(heads, d, dv, dtype, passes):
     """Rows of unequal lengths in one launch, cut into steps (a prompt, portions, single tokens), against the plain
     recurrence over the whole sequence: the state in its slot carries everything; a row without a request writes zeros;
     large gates stay finite through the running maximum. (200 x 200: a state too large for LDS; value heads of 128 and
     256: in bf16 the portions go through the kernel that unrolls the recurrence over chunks of 64 tokens, here with rows
     of less than a chunk, of several chunks and a part, and a state that single tokens have advanced in between.)"""
-    from kestrel_amd.ops import core
+    from kestrel_amd.ops import core, fast
 
+    if passes and (dtype != torch.bfloat16 or not fast.matrix_memory_chunks_scratch(64, 1, heads, d, dv)):
+        pytest.skip("the three passes are the matrix-core kernel's")
     g = _gen(4)
     lengths = [150, 5, 1, 90]
     cap, eps, scale = 6.0, 1e-5, d ** -0.5
@@ -486,9 +489,11 @@ def test_matrix_memory_kernel(heads, d, dv, dtype):
             cu.append(cu[-1] + count)
         x = torch.cat(xs).to(DEV)
         out = torch.full((x.shape[0], heads * dv), 7.0, dtype=dtype, device=DEV)
+        scratch = torch.full((fast.matrix_memory_chunks_scratch(x.shape[0], len(slots), heads, d, dv),), float("nan"),
+                             device=DEV) if passes else None
         core.matrix_memory(x, offsets, torch.cat(pres).to(DEV).contiguous(), state, torch.tensor(cu, dtype=torch.int32, device=DEV),
                            torch.tensor(slots, dtype=torch.int32, device=DEV), gain.to(DEV), out, heads, d, dv, scale, cap, eps,
-                           single_tokens=all(count == 1 for _, count in step), chunks=True)
+                           single_tokens=all(count == 1 for _, count in step), chunks=True, scratch=scratch)
         for i, (r, count) in enumerate(step):
             piece = out[cu[i]:cu[i + 1]].double().cpu()
             if r is None:
