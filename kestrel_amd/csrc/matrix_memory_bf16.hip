@@ -18,7 +18,7 @@
 // those into the state every chunk starts from, m_end = max(F_L + m_start, m_loc),
 // S_end = e^(F_L + m_start - m_end) S_start + e^(m_loc - m_end) S_loc, element by element in fp32 (it also advances the
 // request's state); and every chunk's read-out from its start state, all chunks at once (MC_READ). The passes meet in a
-// buffer of the caller's, per chunk and head S [d, dv], n [d], m and F_L.
+// buffer of the caller's, per chunk and head S [d, dv], n [d], its own maximum, F_L and the maximum it starts from.
 //
 // In turn, a workgroup of four waves per (head, row of the batch) walks over the row's chunks. S^T lives in the accumulators of
 // the state product for the whole walk: wave w owns the value channels [w dv / 4, (w + 1) dv / 4). Operands are staged in
@@ -47,7 +47,7 @@ struct ChunkArgs {
     long out_stride;
     int heads;
     float q_scale, cap, eps;
-    float* chunks;                 // the passes' buffer: fp32 [chunks, heads, d dv + d + 2]
+    float* chunks;                 // the passes' buffer: fp32 [chunks, heads, d dv + d + 3]
     int n_rows;
 };
 
@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
     }
     // where the state comes from and goes to: the request's row (in turn), the chunk's record of the passes' buffer
     float* st = MODE == MC_SEQ ? a.state + ((size_t)slot * a.heads + head) * (D * DV + D + 1)
-                               : a.chunks + ((size_t)blockIdx.y * a.heads + head) * (D * DV + D + 2);
+                               : a.chunks + ((size_t)blockIdx.y * a.heads + head) * (D * DV + D + 3);
     // S^T in accumulators: tile (jb, db), register i of a lane: value channel wave WJ + jb 32 + (i / 4) 8 + half 4 + i % 4,
     // key channel db 32 + col
     mc_floatx16 S[NJ][ND];
@@ -134,7 +134,8 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
                 S[jb][db][i] = MODE == MC_SEQ ? st[(size_t)dd * DV + j] : 0.f;
             }
     for (int e = tid; e < D; e += MC_THREADS) nvec[e] = MODE == MC_LOCAL ? 0.f : st[D * DV + e];
-    float m0 = MODE == MC_LOCAL ? -INFINITY : st[D * DV + D];      // (a chunk as if it started from nothing)
+    // (a chunk as if it started from nothing; a read-out from the maximum that the scan has left for its chunk)
+    float m0 = MODE == MC_LOCAL ? -INFINITY : st[D * DV + D + (MODE == MC_READ ? 2 : 0)];
 
     for (int c0 = first; c0 < t1; c0 += MC_CHUNK) {
         const int valid = min(MC_CHUNK, t1 - c0);
@@ -349,11 +350,14 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_chunk_kernel(ChunkAr
     }
 }
 
-// The scan of the three passes: a workgroup per (head, row). Thread 0 walks over the row's chunks and leaves, per chunk,
-// the two weights of its step and the maximum it starts from; every thread then carries its share of S and n through the
-// chunks, writing into each chunk's record the state it starts from, and the request's state at the end.
+// The scan of the three passes: workgroups per (head, row, slice of the state's numbers). Every workgroup works out the
+// row's chain of maxima from the chunks' records (their own maxima and sums of log forget gates, gathered in parallel)
+// and with it, per chunk, the two weights of its step; every thread then carries its few numbers of S and n through the
+// chunks, writing into each chunk's record the state it starts from, and the request's state at the end. The slice 0
+// workgroup also leaves every chunk the maximum it starts from, and the request's at the end.
+constexpr int MC_SCAN_PER_THREAD = 4;
 __global__ void __launch_bounds__(MC_THREADS) matrix_memory_scan_kernel(ChunkArgs a, int D, int DV) {
-    __shared__ float w_old[MC_SCAN_CHUNKS], w_new[MC_SCAN_CHUNKS];
+    __shared__ float w_old[MC_SCAN_CHUNKS], w_new[MC_SCAN_CHUNKS], m_start[MC_SCAN_CHUNKS];
     const int head = blockIdx.x, r = blockIdx.y, tid = threadIdx.x;
     const int t0 = a.cu_q[r], t1 = a.cu_q[r + 1];
     if (t0 >= t1) return;
@@ -364,23 +368,30 @@ __global__ void __launch_bounds__(MC_THREADS) matrix_memory_scan_kernel(ChunkArg
     const int nc = (t1 - t0 + MC_CHUNK - 1) / MC_CHUNK;
     const int per = D * DV + D;
     float* st = a.state + ((size_t)slot * a.heads + head) * (per + 1);
-    float* rec = a.chunks + ((size_t)base * a.heads + head) * (per + 2);
-    const size_t step = (size_t)a.heads * (per + 2);
+    float* rec = a.chunks + ((size_t)base * a.heads + head) * (per + 3);
+    const size_t step = (size_t)a.heads * (per + 3);
+    for (int c = tid; c < nc; c += MC_THREADS) {
+        w_old[c] = rec[c * step + per + 1];         // (for now: the chunk's sum of log forget gates, and its own maximum)
+        w_new[c] = rec[c * step + per];
+    }
+    __syncthreads();
     if (tid == 0) {
         float m = st[per];
         for (int c = 0; c < nc; ++c) {
-            float* at = rec + c * step;
-            const float m_loc = at[per], f_all = at[per + 1];
+            const float f_all = w_old[c], m_loc = w_new[c];
             const float m_end = fmaxf(f_all + m, m_loc);
             w_old[c] = expf(f_all + m - m_end);
             w_new[c] = expf(m_loc - m_end);
-            at[per] = m;                    // the maximum the chunk starts from
+            m_start[c] = m;
             m = m_end;
         }
-        st[per] = m;
+        if (blockIdx.z == 0) st[per] = m;
     }
     __syncthreads();
-    for (int e = tid; e < per; e += MC_THREADS) {
+    if (blockIdx.z == 0)
+        for (int c = tid; c < nc; c += MC_THREADS) rec[c * step + per + 2] = m_start[c];
+    const int lo = blockIdx.z * MC_THREADS * MC_SCAN_PER_THREAD;
+    for (int e = lo + tid; e < min(per, lo + MC_THREADS * MC_SCAN_PER_THREAD); e += MC_THREADS) {
         float cur = st[e];
         int c = 0;
         for (; c + 3 < nc; c += 4) {        // (four records in flight)
@@ -417,7 +428,7 @@ KA_API int ka_matrix_memory_chunks_supported(int d, int dv) {
 
 // Floats of the passes' buffer for a step of `n` tokens in `n_rows` rows (every row may end in a part of a chunk).
 KA_API long ka_matrix_memory_chunks_scratch(int n, int n_rows, int heads, int d, int dv) {
-    return (long)(n / MC_CHUNK + n_rows) * heads * ((long)d * dv + d + 2);
+    return (long)(n / MC_CHUNK + n_rows) * heads * ((long)d * dv + d + 3);
 }
 
 // chunks != nullptr (of at least ka_matrix_memory_chunks_scratch floats; n = the step's tokens): the three passes;
@@ -439,6 +450,7 @@ KA_API int ka_matrix_memory_chunks_bf16(const void* q, const void* k, const void
     ChunkArgs a{(const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, (const bf16_t*)gate, stride, pre, state, cu_q, row_slot,
                 gain, (bf16_t*)out, out_stride, heads, q_scale, cap, eps, chunks, n_rows};
     const dim3 block(MC_THREADS);
+    const int scan_slices = ka_cdiv((long)d * dv + d, MC_THREADS * MC_SCAN_PER_THREAD);
 #define MC_LAUNCH_MODE(ND, NJ, MODE, GRID)                                                                                  \
     do {                                                                                                                    \
         static bool sized = false;                                                                                          \
@@ -455,7 +467,7 @@ KA_API int ka_matrix_memory_chunks_bf16(const void* q, const void* k, const void
             MC_LAUNCH_MODE(ND, NJ, MC_SEQ, dim3(heads, n_rows));                                                            \
         } else {                                                                                                            \
             MC_LAUNCH_MODE(ND, NJ, MC_LOCAL, dim3(heads, n_chunks));                                                        \
-            hipLaunchKernelGGL(matrix_memory_scan_kernel, dim3(heads, n_rows), block, 0, stream, a, d, dv);                 \
+            hipLaunchKernelGGL(matrix_memory_scan_kernel, dim3(heads, n_rows, scan_slices), block, 0, stream, a, d, dv);    \
             MC_LAUNCH_MODE(ND, NJ, MC_READ, dim3(heads, n_chunks));                                                         \
         }                                                                                                                   \
     }
