@@ -173,6 +173,117 @@ __global__ void __launch_bounds__(MP_THREADS) qkv_prepare_kernel(PrepareArgs a) 
         }
 }
 
+// The same for bf16 rows whose heads are 32, 64 or 128 channels wide: a lane takes eight neighbouring channels with one
+// 16-byte load, LPH lanes a head, so that a wave covers 64 / LPH heads at a time and a head's sum of squares meets inside
+// its lanes. A rotated pair (channels 2i and 2i + 1 only) lies inside a lane's eight. Values in pieces of eight as well.
+typedef __attribute__((ext_vector_type(8))) __bf16 mp_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float mp_floatx4;
+
+template <int LPH>
+__global__ void __launch_bounds__(MP_THREADS) qkv_prepare_wide_kernel(PrepareArgs a) {
+    extern __shared__ float sm[];
+    constexpr int HD = 8 * LPH, HEADS_A_PASS = MP_THREADS / LPH;
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const int group = tid / LPH, sub = tid % LPH;
+    const int heads = a.H + a.G, half = a.rot / 2;
+    float* cs = sm;
+    float* sn = cs + half;
+    float* ss = sn + half;
+    bf16_t* row = reinterpret_cast<bf16_t*>(a.qkv) + (size_t)t * a.row_stride;
+    const int pos = a.positions ? a.positions[t] : 0;
+    if (a.freqs)
+        for (int i = tid; i < half; i += MP_THREADS) sincosf((float)pos * a.freqs[i], &sn[i], &cs[i]);
+    if (a.norm_mode) {
+        for (int h0 = 0; h0 < heads; h0 += HEADS_A_PASS) {
+            const int h = h0 + group;
+            float s = 0.f;
+            if (h < heads) {
+                const mp_bf16x8 x = *reinterpret_cast<const mp_bf16x8*>(row + (size_t)h * HD + sub * 8);
+#pragma unroll
+                for (int u = 0; u < 8; ++u) s += (float)x[u] * (float)x[u];
+            }
+            s = ka_lanes_reduce<1, LPH>(s, KaSum{});
+            if (h < heads && sub == 0) ss[h] = s;
+        }
+    }
+    __syncthreads();
+    float r_all_q = 1.f, r_all_k = 1.f;
+    if (a.norm_mode == 2) {
+        float sq = 0.f, sk = 0.f;
+        for (int h = 0; h < a.H; ++h) sq += ss[h];
+        for (int h = a.H; h < heads; ++h) sk += ss[h];
+        r_all_q = 1.0f / sqrtf(sq / (float)(a.H * HD) + a.eps);
+        r_all_k = 1.0f / sqrtf(sk / (float)(a.G * HD) + a.eps);
+    }
+    const float q_factor = a.q_every > 0 ? 1.0f + a.q_coef * logf((float)((pos + 1) / a.q_every + 1)) : 1.0f;
+    const long slot = a.slots ? a.slots[t] : -1;
+    const long page = slot >= 0 ? slot / a.page_size : 0, off = slot >= 0 ? slot % a.page_size : 0;
+    bf16_t* k_cache = reinterpret_cast<bf16_t*>(a.k_cache);
+    bf16_t* v_cache = reinterpret_cast<bf16_t*>(a.v_cache);
+    for (int h = group; h < heads; h += HEADS_A_PASS) {
+        const bool is_q = h < a.H;
+        if (!is_q && slot < 0) continue;
+        bf16_t* hp = row + (size_t)h * HD + sub * 8;
+        bf16_t* dst = is_q ? hp : k_cache + (((size_t)page * a.G + (h - a.H)) * a.page_size + off) * HD + sub * 8;
+        float r = 1.f;
+        const float* gain = nullptr;
+        if (a.norm_mode == 1) {
+            r = 1.0f / sqrtf(ss[h] / (float)HD + a.eps);
+            gain = is_q ? a.q_gain : a.k_gain;
+        } else if (a.norm_mode == 2) {
+            r = is_q ? r_all_q : r_all_k;
+            gain = is_q ? a.q_gain : a.k_gain;
+            if (gain) gain += (size_t)(is_q ? h : h - a.H) * HD;
+        }
+        const float after = is_q ? q_factor : 1.f;
+        const mp_bf16x8 x = *reinterpret_cast<const mp_bf16x8*>(hp);
+        float y[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) y[u] = (float)x[u] * r;
+        if (gain) {
+            const mp_floatx4 g0 = *reinterpret_cast<const mp_floatx4*>(gain + sub * 8);
+            const mp_floatx4 g1 = *reinterpret_cast<const mp_floatx4*>(gain + sub * 8 + 4);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) { y[u] *= g0[u]; y[4 + u] *= g1[u]; }
+        }
+        if (a.freqs) {
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int i = sub * 4 + p;
+                if (2 * i < a.rot) {
+                    const float u = y[2 * p], v = y[2 * p + 1];
+                    y[2 * p] = u * cs[i] - v * sn[i];
+                    y[2 * p + 1] = v * cs[i] + u * sn[i];
+                }
+            }
+        }
+        mp_bf16x8 o;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) o[u] = (bf16_t)(y[u] * after);
+        *reinterpret_cast<mp_bf16x8*>(dst) = o;
+    }
+    bf16_t* vrow = row + (size_t)heads * HD;
+    const int pieces = a.hdv / 8;
+    const float lam = a.blend == 2 ? *a.lambda : 0.f;
+    bf16_t* other = a.blend ? reinterpret_cast<bf16_t*>(a.v_other) + (size_t)t * a.v_other_stride : nullptr;
+    for (int e = tid; e < a.G * pieces; e += MP_THREADS) {
+        const int g = e / pieces, c0 = (e % pieces) * 8;
+        mp_bf16x8 v = *reinterpret_cast<const mp_bf16x8*>(vrow + (size_t)g * a.hdv + c0);
+        if (a.blend == 1) {
+            *reinterpret_cast<mp_bf16x8*>(other + (size_t)g * a.hdv + c0) = v;
+        } else if (a.blend == 2) {
+            const mp_bf16x8 w = *reinterpret_cast<const mp_bf16x8*>(other + (size_t)g * a.hdv + c0);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = (bf16_t)((1.0f - lam) * (float)v[u] + lam * (float)w[u]);
+        }
+        if (slot >= 0) {
+            bf16_t* vp = v_cache + (((size_t)page * a.G + g) * a.hdv + c0) * a.page_size + off;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) vp[(size_t)u * a.page_size] = v[u];
+        }
+    }
+}
+
 KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* positions, const int* slots, void* k_cache,
                           void* v_cache, int n, int H, int G, int hd, int hdv, int page_size, int norm_mode,
                           const float* q_gain, const float* k_gain, float eps, const float* freqs, int rot, int interleaved,
@@ -197,7 +308,15 @@ KA_API int ka_qkv_prepare(void* qkv, int dtype, long row_stride, const int* posi
     KA_CHECK(lds <= 64 * 1024, "%s: %d heads and %d rotated channels do not fit in LDS", who, H + G, rot);
     PrepareArgs a{qkv, row_stride, positions, slots, k_cache, v_cache, H, G, hd, hdv, page_size, norm_mode, q_gain, k_gain, eps,
                   freqs, rot, interleaved, q_coef, q_every, blend, v_other, v_other_stride, lambda};
-    if (dtype == KA_F32) hipLaunchKernelGGL(qkv_prepare_kernel<float>, dim3(n), dim3(MP_THREADS), lds, stream, a);
+    // bf16 heads of 32, 64 or 128 channels, everything 16-byte aligned, pairs of neighbours if rotated: eight channels a lane
+    const bool wide = dtype == KA_BF16 && (hd == 32 || hd == 64 || hd == 128) && hdv % 8 == 0 && row_stride % 8 == 0 &&
+        (uintptr_t)qkv % 16 == 0 && (freqs == nullptr || interleaved == 1) &&
+        (blend == 0 || ((uintptr_t)v_other % 16 == 0 && v_other_stride % 8 == 0)) &&
+        (uintptr_t)q_gain % 16 == 0 && (uintptr_t)k_gain % 16 == 0 && (slots == nullptr || (uintptr_t)k_cache % 16 == 0);
+    if (wide && hd == 32) hipLaunchKernelGGL(qkv_prepare_wide_kernel<4>, dim3(n), dim3(MP_THREADS), lds, stream, a);
+    else if (wide && hd == 64) hipLaunchKernelGGL(qkv_prepare_wide_kernel<8>, dim3(n), dim3(MP_THREADS), lds, stream, a);
+    else if (wide) hipLaunchKernelGGL(qkv_prepare_wide_kernel<16>, dim3(n), dim3(MP_THREADS), lds, stream, a);
+    else if (dtype == KA_F32) hipLaunchKernelGGL(qkv_prepare_kernel<float>, dim3(n), dim3(MP_THREADS), lds, stream, a);
     else hipLaunchKernelGGL(qkv_prepare_kernel<bf16_t>, dim3(n), dim3(MP_THREADS), lds, stream, a);
     KA_LAUNCH_CHECK();
     return 0;
