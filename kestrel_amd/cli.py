@@ -26,6 +26,9 @@ def _add_runtime_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--kv-cache-pages", type=int, default=None)
     parser.add_argument("--kv-cache-bytes", type=int, default=None, help="size the cache pool by a byte budget instead")
     parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
+    parser.add_argument("--max-seq-len", type=int, default=None,
+                        help="longest sequence a request may grow to (default: what the model allows; a design without a "
+                             "bound of its own names a large number, and captured steps carry block tables of that width)")
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--disable-graphs", action="store_true", help="do not replay steps as HIP graphs")
     parser.add_argument("--pipeline-depth", type=int, default=2, choices=(1, 2),
@@ -62,7 +65,7 @@ def _generate(args) -> int:
     cfg = RuntimeConfig(model_path=args.model_path, model=args.model, device=args.device, dtype=args.dtype,
                         max_batch_size=args.max_batch_size, page_size=args.page_size,
                         kv_cache_pages=args.kv_cache_pages, kv_cache_bytes=args.kv_cache_bytes,
-                        max_num_batched_tokens=args.max_num_batched_tokens,
+                        max_num_batched_tokens=args.max_num_batched_tokens, max_seq_len=args.max_seq_len,
                         seed=args.seed, enable_graphs=not args.disable_graphs, pipeline_depth=args.pipeline_depth,
                         warmup=not args.no_warmup, tune_linears=args.tune_linears)
     engine = InferenceEngine.create_sync(cfg)

@@ -308,6 +308,32 @@ def test_trace_replay_program(dtype, tmp_path):
             _close(got[row:row + 1], want[row:row + 1], run_dtype, f"trace step {step} {tag}[{p}]", folder, ids[tag], rows=[p])
 
 
+def test_command_line(tmp_path):
+    """``python -m kestrel_amd random-weights`` from a configuration of this design, then ``generate`` on the folder."""
+    import sys
+
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    config = tmp_path / "cfg.json"
+    config.write_text(json.dumps(cases.CONFIGS["S"]))
+    made = subprocess.run([sys.executable, "-m", "kestrel_amd", "random-weights", "--out", str(tmp_path / "m"), "--config", str(config),
+                           "--seed", "5", "--std", "0.08", "--bias-std", "0.5", "--gain-std", "0.2"], capture_output=True, text=True,
+                          env=env, cwd=ROOT)
+    assert made.returncode == 0, made.stderr
+    folder = str(tmp_path / "m")
+    prompt = _ids(folder, 990, 9)
+    done = subprocess.run([sys.executable, "-m", "kestrel_amd", "generate", "--model-path", folder, "--dtype", "float32",
+                           "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "6", "--temperature", "0",
+                           "--kv-cache-pages", "8", "--max-seq-len", "64"], capture_output=True, text=True, env=env, cwd=ROOT,
+                          timeout=300)
+    assert done.returncode == 0, done.stderr
+    tokens = json.loads(done.stdout.strip().splitlines()[-1])["tokens"]
+    assert len(tokens) == 6
+    logits = plain.forward(cases.config_of(folder), cases.stored_weights(folder), prompt + tokens[:-1])
+    for i, token in enumerate(tokens):
+        row = logits[len(prompt) - 1 + i]
+        assert float(row.max() - row[token]) <= 1e-4 * max(1.0, float(row.std())), f"token {i}"
+
+
 # ------------------------------------------------------------------------------------------------ each mechanism's kernel alone
 def _gen(seed):
     return torch.Generator().manual_seed(seed)
