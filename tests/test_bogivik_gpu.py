@@ -460,10 +460,13 @@ def test_gate_and_branches_kernels(dtype):
         assert torch.allclose(out.double().cpu(), base.double() + 2.0 * plain.rms_norm(a.double(), None, 1e-5), rtol=2e-5, atol=2e-5)
 
 
-@pytest.mark.parametrize("passes", [False, True], ids=["in turn", "three passes"])
-@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
-@pytest.mark.parametrize("heads, d, dv", [(3, 20, 36), (1, 8, 300), (2, 64, 64), (2, 200, 200), (2, 64, 128), (1, 32, 256),
-                                          (1, 128, 128), (3, 64, 256)])
+_MEMORY_SIZES = [(3, 20, 36), (1, 8, 300), (2, 64, 64), (2, 200, 200), (2, 64, 128), (1, 32, 256), (1, 128, 128), (3, 64, 256)]
+
+
+@pytest.mark.parametrize("heads, d, dv, dtype, passes",
+                         [(*size, dtype, False) for size in _MEMORY_SIZES for dtype in DTYPES]
+                         + [(*size, torch.bfloat16, True) for size in _MEMORY_SIZES if size[1] in (32, 64, 128) and size[2] in (128, 256)],
+                         ids=lambda v: {torch.float32: "fp32", torch.bfloat16: "bf16", True: "three passes", False: "in turn"}.get(v, str(v)))
 def test_matrix_memory_kernel(heads, d, dv, dtype, passes):
     """Rows of unequal lengths in one launch, cut into steps (a prompt, portions, single tokens), against the plain
     recurrence over the whole sequence: the state in its slot carries everything; a row without a request writes zeros;
@@ -472,8 +475,7 @@ def test_matrix_memory_kernel(heads, d, dv, dtype, passes):
     of less than a chunk, of several chunks and a part, and a state that single tokens have advanced in between.)"""
     from kestrel_amd.ops import core, fast
 
-    if passes and (dtype != torch.bfloat16 or not fast.matrix_memory_chunks_scratch(64, 1, heads, d, dv)):
-        pytest.skip("the three passes are the matrix-core kernel's")
+    assert not passes or fast.matrix_memory_chunks_scratch(64, 1, heads, d, dv), "the three passes do not cover these sizes"
     g = _gen(4)
     lengths = [150, 5, 1, 90]
     cap, eps, scale = 6.0, 1e-5, d ** -0.5
