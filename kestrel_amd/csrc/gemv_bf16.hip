@@ -464,6 +464,7 @@ static int launch_split(int waves, int strips, hipStream_t stream, const SkinnyA
 // LayerNorm(ln_x) (M <= 16, K1 <= 2048). Target b (Wb non-null) shares the input.
 struct SkinnyExtras {                 // what only some callers of skinny_fused bring
     const KaThenNorm* then = nullptr; // a norm of the finished rows
+    bool ln_uncentred = false;        // the norm of the prologue takes no mean off: x / sqrt(mean(x^2) + eps) * gamma
     void* ln_store = nullptr;         // where the LayerNorm prologue also leaves its normalised rows (bf16)
     long ln_store_ld = 0;
 };
@@ -501,6 +502,7 @@ static int skinny_fused(const SkinnyExtras& extras, const void* A1, long lda1, i
                      (uintptr_t)ln_beta % 16 == 0, "%s: LayerNorm operands must be 16-byte aligned", who);
         KA_CHECK(A2 == nullptr && !accumulate_a, "%s: no second segment and no accumulation with a LayerNorm prologue", who);
         args.ln_x = ln_x; args.ln_gamma = ln_gamma; args.ln_beta = ln_beta; args.ln_eps = ln_eps;
+        args.ln_uncentred = extras.ln_uncentred ? 1 : 0;
         if (extras.ln_store) {
             KA_CHECK(extras.ln_store_ld >= K1 && extras.ln_store_ld % 8 == 0 && (uintptr_t)extras.ln_store % 16 == 0,
                      "%s: the stored normalised rows must be 16-byte aligned and >= K apart", who);
@@ -631,6 +633,20 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     return skinny_fused(SkinnyExtras{}, A1, lda1, K1, A2, lda2, K2, W2, ldw2, bias2, ln_x, ln_gamma, ln_beta, ln_eps, Wa, ldwa, biasa,
                         outa, out_dtype_a, ldoa, Na, acta, accumulate_a, Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, M,
                         target_waves, partials, partial_floats, stream);
+}
+
+// The same with a root-mean-square norm as the prologue: h = x / sqrt(mean(x^2) + eps) * gamma (no mean, no shift).
+KA_API int ka_linear_skinny_fused_rms(const float* ln_x, const float* ln_gamma, float ln_eps, int K1, const void* Wa,
+                                      long ldwa, const float* biasa, void* outa, int out_dtype_a, long ldoa, int Na,
+                                      int acta, const void* Wb, long ldwb, const float* biasb, void* outb,
+                                      int out_dtype_b, long ldob, int Nb, int actb, int M, int target_waves,
+                                      hipStream_t stream) {
+    KA_CHECK(ln_x != nullptr, "ka_linear_skinny_fused_rms: rows to normalise missing");
+    SkinnyExtras extras;
+    extras.ln_uncentred = true;
+    return skinny_fused(extras, nullptr, 0, K1, nullptr, 0, 0, nullptr, 0, nullptr, ln_x, ln_gamma, nullptr, ln_eps, Wa, ldwa,
+                        biasa, outa, out_dtype_a, ldoa, Na, acta, 0, Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, M,
+                        target_waves, nullptr, 0, stream);
 }
 
 // out (+)= A1 W1^T + b1 + A2 W2^T + b2 into fp32 rows, then normed = LayerNorm(out; gamma, beta, eps):

@@ -87,6 +87,7 @@ struct SkinnyArgs {
     const float* ln_gamma;
     const float* ln_beta;
     float ln_eps;
+    int ln_uncentred;       // the prologue divides by the root mean square and takes no mean off (an RMS norm)
     bf16_t* ln_store;       // non-null: workgroup 0 also stores the normalised rows here, [M, K[0]] rows ln_store_ld apart
     long ln_store_ld;
     SkinnyTarget a, b;      // b.W null: one target
@@ -192,7 +193,7 @@ __device__ __forceinline__ void sk_normalise_row(const SkinnyArgs& p, bf16_t* xs
         if ((j * KA_WAVE + lane) * 4 >= K) row.x[j] = floatx4{0.f, 0.f, 0.f, 0.f};
         s += (row.x[j][0] + row.x[j][1]) + (row.x[j][2] + row.x[j][3]);
     }
-    float mean = ka_wave_sum(s) / (float)K;
+    float mean = p.ln_uncentred ? 0.f : ka_wave_sum(s) / (float)K;
     float q = 0.f;
 #pragma unroll
     for (int j = 0; j < XV; ++j) {

@@ -111,9 +111,13 @@ class DecoderModel:
         """A few decoded rows, every one of them wanted, in order: the head's launch normalises them itself
         (one launch less a step)."""
         ln = self.final_norm.layernorm_operands()
-        if self.dtype != torch.bfloat16 or not batch.decode_only or not getattr(batch, "wants_every_token", False) or ln is None:
+        rms = self.final_norm.rms_operands() if ln is None and callable(getattr(self.final_norm, "rms_operands", None)) else None
+        if self.dtype != torch.bfloat16 or not batch.decode_only or not getattr(batch, "wants_every_token", False) \
+                or (ln is None and rms is None):
             return False
         from ..ops import fast
+        if ln is None:
+            return fast.layernorm_linear(x, rms[0], None, rms[1], self.head_weight, self.head_bias, logits, 0, centred=False)
         return fast.layernorm_linear(x, *ln, self.head_weight, self.head_bias, logits, 0)
 
     # ------------------------------------------------------------------ forward

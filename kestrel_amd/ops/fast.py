@@ -26,6 +26,9 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_int,   # target a
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int,           # target b
         _c_int, _c_int, _c_void_p, _c_long, _c_void_p],               # M, target_waves, partial sums and how many, stream
+    "ka_linear_skinny_fused_rms": [_c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long,
+                                   _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_int,
+                                   _c_int, _c_void_p],
     "ka_linear_skinny_pair_norm": [
         _c_void_p, _c_long, _c_int, _c_void_p, _c_long, _c_int,                  # A1, lda1, K1, A2, lda2, K2
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_long, _c_void_p,            # W1, ldw1, bias1, W2, ldw2, bias2
@@ -368,11 +371,16 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
     return True
 
 
-def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None, out_b=None, act_b=0, store=None) -> bool:
+def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None, out_b=None, act_b=0, store=None,
+                     centred: bool = True) -> bool:
     """``h = LayerNorm(x)``; ``out_a = act_a(h @ wa.T + ba)`` and, if a second target is given,
     ``out_b = act_b(h @ wb.T + bb)`` in one launch: the kernel normalises the fp32 rows itself
     (at most 16 of them, at most 4096 wide, and no more than fit in 96 KB of LDS as bf16).
-    ``store`` (one target only): bf16 ``[m, k]`` that also receives ``h``, for launches that follow."""
+    ``store`` (one target only): bf16 ``[m, k]`` that also receives ``h``, for launches that follow.
+    ``centred`` ``False``: the norm is a root-mean-square norm, ``h = x / sqrt(mean(x^2) + eps) * gamma`` (no ``beta``,
+    no ``store``)."""
+    if not centred and (beta is not None or store is not None):
+        return False
     m, k = x.shape
     if not (0 < m <= SKINNY_LN_MAX_ROWS) or k % 8 or k > SKINNY_LN_MAX_WIDTH or x.dtype != torch.float32 \
             or not x.is_contiguous():
@@ -400,6 +408,13 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
             x.data_ptr(), gamma.data_ptr(), _ptr(beta), float(eps), k, wa.data_ptr(), wa.stride(0), _ptr(ba),
             out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, m, store.data_ptr(), store.stride(0),
             stream_ptr()))
+        return True
+    if not centred:
+        _check(lib().ka_linear_skinny_fused_rms(
+            x.data_ptr(), gamma.data_ptr(), float(eps), k, wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(),
+            _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, _ptr(wb), wb.stride(0) if two else 0, _ptr(bb) if two else None,
+            _ptr(out_b), _OUT_CODE[out_b.dtype] if two else 0, out_b.stride(0) if two else 0, nb, act_b, m,
+            chip_sizes(x.device).skinny_target_waves, stream_ptr()))
         return True
     _check(lib().ka_linear_skinny_fused(
         None, 0, k, None, 0, 0, None, 0, None,

@@ -54,6 +54,12 @@ class Norm(Part):
         ``None`` (the default): the norm is always run through ``forward``, in a launch of its own."""
         return None
 
+    def rms_operands(self):
+        """Optional. A norm that computes ``x / sqrt(mean(x^2) + eps) * weight`` over the last axis says so here:
+        ``(weight fp32 [dim], eps)``; a block's first norm and the final norm are then taken into the launch of
+        the linear behind them in decode steps of a few rows. ``None`` (the default): not such a norm."""
+        return None
+
 
 @dataclass(frozen=True)
 class Rotation:

@@ -36,6 +36,11 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
     if normed is not None:
         fused = fast.linear_two_outputs(normed, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3])
     ln = norm.layernorm_operands()            # (a norm of another form is run through its own forward below)
+    rms = norm.rms_operands() if ln is None and callable(getattr(norm, "rms_operands", None)) else None
+    if not fused and fast.FUSE_LAYERNORM_PROLOGUE and rms is not None:
+        # a root-mean-square norm in the prologue of the launch that projects for the mixer and the feed-forward
+        fused = fast.layernorm_linear(x, rms[0], None, rms[1], m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3],
+                                      centred=False)
     if not fused and fast.FUSE_LAYERNORM_PROLOGUE and ln is not None:
         # the feed-forward's first linear goes into the mixer's launch where the mixer takes it (the
         # launch of the mixer's first linear then leaves the normalised rows for it), else into the

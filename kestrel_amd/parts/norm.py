@@ -45,8 +45,8 @@ class LayerNorm(Norm):
 
 class RMSNorm(Norm):
     """``x / sqrt(mean(x^2) + eps) * weight`` over the last axis: no mean is taken off, no shift is added, the
-    weight is used as stored (not as one plus it). It offers no ``layernorm_operands``, so it always runs in a
-    launch of its own."""
+    weight is used as stored (not as one plus it). It offers no ``layernorm_operands`` (it is no LayerNorm), but
+    ``rms_operands``: the weight-streaming linears of a few rows take it into their launch as they take a LayerNorm."""
 
     replays_every_step = True
 
@@ -62,6 +62,10 @@ class RMSNorm(Norm):
 
     def forward(self, x, out, rows=None) -> None:
         core.rmsnorm(x, self.weight, self.spec.eps, out, rows)
+
+    def rms_operands(self):
+        """``(weight fp32 [dim], eps)`` of ``x / sqrt(mean(x^2) + eps) * weight``."""
+        return self.weight, float(self.spec.eps)
 
 
 register_norm("layernorm", LayerNorm)
